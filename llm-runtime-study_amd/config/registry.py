@@ -72,10 +72,14 @@ def _load_builtin() -> None:
     _builtin_loaded = True
     from ..models.qwen3 import build_spec
     from ..text.chat import format_qwen3_chat
+    from ..models.nobodra import build_spec as build_nobodra
+    from .nobodra import NobodraConfig
     from .qwen3 import Qwen3Config
 
     if Qwen3Config.ARCHITECTURE not in _ARCHITECTURES:
         register_architecture(Qwen3Config.ARCHITECTURE, Qwen3Config, build_spec, chat_template=format_qwen3_chat)
+    if NobodraConfig.ARCHITECTURE not in _ARCHITECTURES:
+        register_architecture(NobodraConfig.ARCHITECTURE, NobodraConfig, build_nobodra)      # token ids only: it has no chat template
     import importlib
     import os
 
@@ -107,8 +111,10 @@ def registered_architectures() -> tuple[str, ...]:
 
 def architecture_for(raw: dict) -> Architecture:
     names = raw.get("architectures")
+    if names is None and isinstance(raw.get("architecture"), str):
+        names = [raw["architecture"]]         # some configurations name their one architecture as a plain string
     if not isinstance(names, list) or len(names) != 1 or not isinstance(names[0], str):
-        raise ConfigError(f"config.json must name exactly one architecture in `architectures`, got {names!r}")
+        raise ConfigError(f"config.json must name exactly one architecture in `architectures` (or `architecture`), got {names!r}")
     _load_builtin()
     try:
         return _ARCHITECTURES[names[0]]

@@ -813,3 +813,42 @@ LRS_API int lrs_gather_rows(float* out, const float* x, const int* rows, int n_r
   gather_rows_kernel<<<n_rows, 256, 0, (hipStream_t)stream>>>(out, x, rows, hidden);
   return lrs_check_launch("gather_rows");
 }
+
+// ------------------------------------------------ norm of a sublayer's output, added to the stream
+// residual[r] += w * y[r] * rsqrt(mean(y[r]^2) + eps), all float32: the layer arrangement that normalises what a
+// mixer or feed-forward gives out rather than what it is given.
+template <typename TW>
+__global__ __launch_bounds__(256) void norm_add_kernel(float* __restrict__ residual, const float* __restrict__ y,
+                                                       const TW* __restrict__ weight, int hidden, float eps) {
+  __shared__ float scratch[16];
+  const float* src = y + (int64_t)blockIdx.x * hidden;
+  float* dst = residual + (int64_t)blockIdx.x * hidden;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) ss = fmaf(src[i], src[i], ss);
+  ss = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)hidden + eps);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] += to_float(weight[i]) * (src[i] * inv);
+}
+LRS_API int lrs_norm_add(float* residual, const float* y, const void* weight, int w_dtype, int n_rows, int hidden, float eps,
+                         void* stream) {
+  LRS_REQUIRE(n_rows > 0 && hidden > 0 && eps > 0.f, "norm_add: bad sizes rows=%d hidden=%d", n_rows, hidden);
+  if (w_dtype == LRS_F32) norm_add_kernel<float><<<n_rows, 256, 0, (hipStream_t)stream>>>(residual, y, (const float*)weight, hidden, eps);
+  else if (w_dtype == LRS_BF16) norm_add_kernel<bf16><<<n_rows, 256, 0, (hipStream_t)stream>>>(residual, y, (const bf16*)weight, hidden, eps);
+  else return lrs_fail("norm_add: unknown weight dtype %d", w_dtype);
+  return lrs_check_launch("norm_add");
+}
+
+// ------------------------------------------------ the float32 stream as an activation
+// out = x rounded to the activation dtype, for sublayers that read the residual stream itself.
+template <typename TO>
+__global__ void round_rows_kernel(TO* __restrict__ out, const float* __restrict__ x, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) out[i] = from_float<TO>(x[i]);
+}
+LRS_API int lrs_round_rows(void* out, int out_dtype, const float* x, int64_t n, void* stream) {
+  LRS_REQUIRE(n > 0, "round_rows: nothing to do");
+  const int blocks = (int)((n + 1023) / 1024 < 4096 ? (n + 1023) / 1024 : 4096);
+  if (out_dtype == LRS_BF16) round_rows_kernel<bf16><<<blocks, 256, 0, (hipStream_t)stream>>>((bf16*)out, x, n);
+  else if (out_dtype == LRS_F32) round_rows_kernel<float><<<blocks, 256, 0, (hipStream_t)stream>>>((float*)out, x, n);
+  else return lrs_fail("round_rows: unknown dtype %d", out_dtype);
+  return lrs_check_launch("round_rows");
+}

@@ -1,0 +1,349 @@
+// Routed experts: every token runs `top` of `experts` small feed-forward layers and adds their outputs up,
+// weighted by a softmax over the chosen router logits.
+//
+//   moe_route     per token: the `top` largest of (router logits + bias), lowest index first among equals, and
+//                 the softmax over those alone (float32);
+//   moe_align     one workgroup: sorts the step's (token, choice) pairs by expert into runs padded to whole row
+//                 tiles, so that every tile of the two products below belongs to one expert.  The number of tiles
+//                 a launch is sized for follows from the step's shape alone (pairs / tile + experts at most), so a
+//                 step can be recorded or captured; tiles beyond the ones in use leave at once;
+//   moe_experts   the grouped product: rows gathered through the sorted list, an expert's matrix per tile, and
+//                 optionally the activation (the square of relu) on the way out.  A float32 / any-shape form on
+//                 the vector units, whose sums over K run in one order whatever else is in the step, and a
+//                 bfloat16 form on the matrix cores;
+//   moe_combine   per token: the weighted sum of its experts' rows in the order of its choices, and, when a norm
+//                 weight is given, the RMS norm of that sum added into the residual stream.
+#include "common.h"
+
+namespace {
+
+constexpr int ROUTE_MAX_PER_LANE = 8;     // experts up to 64 * 8
+
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int ld, const float* __restrict__ bias,
+                                                        int* __restrict__ ids, float* __restrict__ weights, int tokens,
+                                                        int experts, int top) {
+  const int t = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  if (t >= tokens) return;
+  float v[ROUTE_MAX_PER_LANE];
+#pragma unroll
+  for (int c = 0; c < ROUTE_MAX_PER_LANE; ++c) {
+    const int e = lane + WAVE * c;
+    v[c] = e < experts ? logits[(int64_t)t * ld + e] + (bias ? bias[e] : 0.f) : -INFINITY;
+  }
+  float first = 0.f, mine = 0.f, total = 0.f;
+  int chosen = 0;
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY;
+#pragma unroll
+    for (int c = 0; c < ROUTE_MAX_PER_LANE; ++c) best = fmaxf(best, v[c]);
+    best = wave_max(best);
+    int where = 1 << 30;
+#pragma unroll
+    for (int c = ROUTE_MAX_PER_LANE - 1; c >= 0; --c)
+      if (v[c] == best) where = lane + WAVE * c;
+#pragma unroll
+    for (int off = WAVE / 2; off > 0; off >>= 1) where = min(where, __shfl_xor(where, off, WAVE));
+    if (where >= experts) where = k;    // logits that are not numbers: any expert, never an index outside the table
+#pragma unroll
+    for (int c = 0; c < ROUTE_MAX_PER_LANE; ++c)
+      if (lane + WAVE * c == where) v[c] = -INFINITY;
+    if (k == 0) first = best;
+    const float w = expf(best - first);
+    total += w;
+    if (lane == k % WAVE && k / WAVE == 0) {
+      mine = w;
+      chosen = where;
+    }
+    if (k >= WAVE) {                    // more choices than lanes: written as they come, scaled below
+      if (lane == 0) {
+        ids[(int64_t)t * top + k] = where;
+        weights[(int64_t)t * top + k] = w;
+      }
+    }
+  }
+  if (lane < top && lane < WAVE) {
+    ids[(int64_t)t * top + lane] = chosen;
+    weights[(int64_t)t * top + lane] = mine / total;
+  }
+  if (top > WAVE && lane == 0)
+    for (int k = WAVE; k < top; ++k) weights[(int64_t)t * top + k] /= total;
+}
+
+// sorted [capacity]: the pair (token * top + choice) at each row of the sorted order, -1 for the rows that pad an
+// expert's run to whole tiles; place [pairs]: the row of each pair; tile_expert [max_tiles]: the expert of each
+// tile of `tile` rows, -1 for tiles not in use.
+__global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__ ids, int pairs, int experts, int tile,
+                                                         int* __restrict__ sorted, int capacity, int* __restrict__ place,
+                                                         int* __restrict__ tile_expert, int max_tiles) {
+  extern __shared__ int shared[];
+  int* count = shared;                  // [experts]
+  int* first = count + experts;         // [experts + 1]: first row of each expert's run
+  int* cursor = first + experts + 1;    // [experts]
+  const int tid = threadIdx.x;
+  for (int e = tid; e < experts; e += blockDim.x) count[e] = cursor[e] = 0;
+  for (int i = tid; i < capacity; i += blockDim.x) sorted[i] = -1;
+  for (int i = tid; i < max_tiles; i += blockDim.x) tile_expert[i] = -1;
+  __syncthreads();
+  for (int i = tid; i < pairs; i += blockDim.x) atomicAdd(&count[min((unsigned)ids[i], (unsigned)experts - 1)], 1);
+  __syncthreads();
+  if (tid == 0) {
+    int at = 0;
+    for (int e = 0; e < experts; ++e) {
+      first[e] = at;
+      at += (count[e] + tile - 1) / tile * tile;
+    }
+    first[experts] = at;
+  }
+  __syncthreads();
+  for (int e = tid; e < experts; e += blockDim.x)
+    for (int i = first[e] / tile; i < first[e + 1] / tile; ++i) tile_expert[i] = e;
+  for (int i = tid; i < pairs; i += blockDim.x) {
+    const int e = min((unsigned)ids[i], (unsigned)experts - 1), row = first[e] + atomicAdd(&cursor[e], 1);
+    sorted[row] = i;
+    place[i] = row;
+  }
+}
+
+enum { ACT_NONE = 0, ACT_RELU_SQUARED = 1 };
+
+// Any dtype, any shape: a 32 x 64 tile of outputs per workgroup of 256 threads, a thread 2 x 4 of them, each the
+// sum of its products in the order of k.
+template <typename T, typename TO>
+__global__ __launch_bounds__(256) void moe_experts_kernel(TO* __restrict__ out, int ldc, const T* __restrict__ a, int lda,
+                                                          const T* __restrict__ w, int n, int k, const int* __restrict__ sorted,
+                                                          const int* __restrict__ tile_expert, int top, int gather, int act) {
+  constexpr int TM = 32, TN = 64, TK = 16;
+  const int expert = tile_expert[blockIdx.x];
+  if (expert < 0) return;
+  __shared__ float a_s[TK][TM + 1];
+  __shared__ float b_s[TK][TN + 1];
+  __shared__ int row_of[TM];
+  const int tid = threadIdx.x, row0 = blockIdx.x * TM, col0 = blockIdx.y * TN;
+  if (tid < TM) {
+    const int pair = sorted[row0 + tid];
+    row_of[tid] = pair < 0 ? -1 : (gather ? pair / top : row0 + tid);
+  }
+  __syncthreads();
+  const T* we = w + (int64_t)expert * n * k;
+  const int ty = tid / 16, tx = tid % 16;
+  float acc[2][4] = {};
+  for (int k0 = 0; k0 < k; k0 += TK) {
+    for (int e = tid; e < TM * TK; e += 256) {
+      const int m = e / TK, kk = e % TK, src = row_of[m];
+      a_s[kk][m] = (src >= 0 && k0 + kk < k) ? to_float(a[(int64_t)src * lda + k0 + kk]) : 0.f;
+    }
+    for (int e = tid; e < TN * TK; e += 256) {
+      const int c = e / TK, kk = e % TK;
+      b_s[kk][c] = (col0 + c < n && k0 + kk < k) ? to_float(we[(int64_t)(col0 + c) * k + k0 + kk]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < TK; ++kk) {
+      float av[2], bv[4];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) av[i] = a_s[kk][ty * 2 + i];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) bv[i] = b_s[kk][tx * 4 + i];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) acc[i][jj] = fmaf(av[i], bv[jj], acc[i][jj]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int m = ty * 2 + i;
+    if (row_of[m] < 0) continue;
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+      const int c = col0 + tx * 4 + jj;
+      if (c >= n) continue;
+      float v = acc[i][jj];
+      if (act == ACT_RELU_SQUARED) v = v > 0.f ? v * v : 0.f;
+      out[(int64_t)(row0 + m) * ldc + c] = from_float<TO>(v);
+    }
+  }
+}
+
+// bfloat16 on the matrix cores: a workgroup of four waves makes 32 rows x 128 columns of one expert, a wave 32 x 32
+// as two by two products of 16 x 16 x 32; K in slices of 64 through LDS, rows padded by 8 values so that the
+// 16-byte fragment reads of a wave fall on different banks; the next slice is read into registers while one is
+// multiplied.
+constexpr int GM = 32, GN = 128, GK = 64, GPAD = 8;
+
+template <typename TO>
+__global__ __launch_bounds__(256) void moe_experts_bf16_kernel(TO* __restrict__ out, int ldc, const bf16* __restrict__ a, int lda,
+                                                               const bf16* __restrict__ w, int n, int k, const int* __restrict__ sorted,
+                                                               const int* __restrict__ tile_expert, int top, int gather, int act) {
+  const int expert = tile_expert[blockIdx.x];
+  if (expert < 0) return;
+  __shared__ __attribute__((aligned(16))) bf16 a_s[GM][GK + GPAD];
+  __shared__ __attribute__((aligned(16))) bf16 b_s[GN][GK + GPAD];
+  __shared__ int row_of[GM];
+  const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+  const int row0 = blockIdx.x * GM, col0 = blockIdx.y * GN;
+  if (tid < GM) {
+    const int pair = sorted[row0 + tid];
+    row_of[tid] = pair < 0 ? -1 : (gather ? pair / top : row0 + tid);
+  }
+  __syncthreads();
+  const bf16* we = w + (int64_t)expert * n * k;
+  // a thread brings 8 values (16 bytes) of one row of the slice: 32 x 64 of the rows is one piece each, 128 x 64 of the
+  // weights four
+  const int a_row = tid / 8, a_col = (tid % 8) * 8;
+  const int a_src = row_of[a_row];
+  const bf16* a_ptr = a_src >= 0 ? a + (int64_t)a_src * lda + a_col : nullptr;
+  bf16x8 a_reg, b_reg[4];
+  const bf16x8 zero = {};
+  auto fetch = [&](int k0) {
+    a_reg = a_ptr ? *(const bf16x8*)(a_ptr + k0) : zero;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const int r = p * 32 + a_row;
+      b_reg[p] = col0 + r < n ? *(const bf16x8*)(we + (int64_t)(col0 + r) * k + k0 + a_col) : zero;
+    }
+  };
+  floatx4 acc[2][2] = {};
+  fetch(0);
+  const int frag_row = lane % 16, frag_k = (lane / 16) * 8;
+  for (int k0 = 0; k0 < k; k0 += GK) {
+    *(bf16x8*)&a_s[a_row][a_col] = a_reg;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) *(bf16x8*)&b_s[p * 32 + a_row][a_col] = b_reg[p];
+    __syncthreads();
+    if (k0 + GK < k) fetch(k0 + GK);
+#pragma unroll
+    for (int kk = 0; kk < GK; kk += 32) {
+      bf16x8 af[2], bfr[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) af[i] = *(const bf16x8*)&a_s[i * 16 + frag_row][kk + frag_k];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) bfr[i] = *(const bf16x8*)&b_s[wave * 32 + i * 16 + frag_row][kk + frag_k];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj)
+          // the weights as the first operand: a lane then holds four consecutive columns of one output row
+          acc[i][jj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bfr[jj], af[i], acc[i][jj], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+  // lane l of a product holds output row (l % 16) and columns (l / 16) * 4 .. + 4 of its 16 x 16
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int m = i * 16 + lane % 16;
+    if (row_of[m] < 0) continue;
+#pragma unroll
+    for (int jj = 0; jj < 2; ++jj) {
+      const int c = col0 + wave * 32 + jj * 16 + (lane / 16) * 4;
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        if (c + x >= n) continue;
+        float v = acc[i][jj][x];
+        if (act == ACT_RELU_SQUARED) v = v > 0.f ? v * v : 0.f;
+        out[(int64_t)(row0 + m) * ldc + c + x] = from_float<TO>(v);
+      }
+    }
+  }
+}
+
+template <typename TW>
+__global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ residual, const float* __restrict__ rows, int hidden,
+                                                          const int* __restrict__ place, const float* __restrict__ weights, int top,
+                                                          const TW* __restrict__ norm_w, float eps) {
+  extern __shared__ float sum[];        // [hidden], then 16 floats for the reduction
+  const int t = blockIdx.x;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float acc = 0.f;
+    for (int c = 0; c < top; ++c)
+      acc = fmaf(weights[(int64_t)t * top + c], rows[(int64_t)place[(int64_t)t * top + c] * hidden + i], acc);
+    sum[i] = acc;
+    ss = fmaf(acc, acc, ss);
+  }
+  float* out = residual + (int64_t)t * hidden;
+  if (!norm_w) {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) out[i] += sum[i];
+    return;
+  }
+  ss = block_sum(ss, sum + hidden);
+  const float inv = 1.0f / sqrtf(ss / (float)hidden + eps);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) out[i] += sum[i] * inv * to_float(norm_w[i]);
+}
+
+}  // namespace
+
+LRS_API int lrs_moe_tile_rows() { return 32; }
+
+// The most tiles that `pairs` (token, choice) pairs of `experts` experts can fill: every expert in use ends in at
+// most one tile that is not full.
+LRS_API int lrs_moe_max_tiles(int pairs, int experts) {
+  const int padded = pairs / lrs_moe_tile_rows() + experts;
+  return pairs < padded ? pairs : padded;
+}
+
+LRS_API int lrs_moe_route(const float* logits, int ld, const float* bias, int* ids, float* weights, int tokens, int experts,
+                          int top, void* stream) {
+  LRS_REQUIRE(tokens > 0 && experts > 0 && top > 0 && top <= experts, "moe_route: bad sizes tokens=%d experts=%d top=%d", tokens, experts, top);
+  LRS_REQUIRE(experts <= WAVE * ROUTE_MAX_PER_LANE, "moe_route: at most %d experts, got %d", WAVE * ROUTE_MAX_PER_LANE, experts);
+  LRS_REQUIRE(ld >= experts, "moe_route: rows of %d logits hold fewer than %d experts", ld, experts);
+  moe_route_kernel<<<(tokens + 3) / 4, 256, 0, (hipStream_t)stream>>>(logits, ld, bias, ids, weights, tokens, experts, top);
+  return lrs_check_launch("moe_route");
+}
+
+LRS_API int lrs_moe_align(const int* ids, int pairs, int experts, int* sorted, int capacity, int* place, int* tile_expert,
+                          int max_tiles, void* stream) {
+  const int tile = lrs_moe_tile_rows();
+  LRS_REQUIRE(pairs > 0 && experts > 0, "moe_align: bad sizes pairs=%d experts=%d", pairs, experts);
+  LRS_REQUIRE(max_tiles >= lrs_moe_max_tiles(pairs, experts), "moe_align: %d tiles may not hold %d pairs of %d experts", max_tiles, pairs, experts);
+  LRS_REQUIRE(capacity >= max_tiles * tile, "moe_align: the sorted list holds %d rows, %d tiles need %d", capacity, max_tiles, max_tiles * tile);
+  const size_t lds = (size_t)(3 * experts + 1) * sizeof(int);
+  LRS_REQUIRE(lds <= 48 * 1024, "moe_align: %d experts are too many", experts);
+  moe_align_kernel<<<1, 1024, lds, (hipStream_t)stream>>>(ids, pairs, experts, tile, sorted, capacity, place, tile_expert, max_tiles);
+  return lrs_check_launch("moe_align");
+}
+
+// out [max_tiles * tile, n] = rows of `a` (row pair / top of the sorted list if `gather`, else the sorted row
+// itself) times the tile's expert matrix w[expert] [n, k], transposed; act 1: the square of relu.
+LRS_API int lrs_moe_experts(void* out, int out_dtype, int ldc, const void* a, const void* w, int dtype, int lda, int n, int k,
+                            const int* sorted, const int* tile_expert, int max_tiles, int top, int gather, int act, void* stream) {
+  LRS_REQUIRE(max_tiles > 0 && n > 0 && k > 0 && top > 0, "moe_experts: bad sizes tiles=%d n=%d k=%d top=%d", max_tiles, n, k, top);
+  LRS_REQUIRE(lda >= k && ldc >= n, "moe_experts: strides lda=%d ldc=%d too small for k=%d n=%d", lda, ldc, k, n);
+  LRS_REQUIRE(act == ACT_NONE || act == ACT_RELU_SQUARED, "moe_experts: unknown activation %d", act);
+  hipStream_t s = (hipStream_t)stream;
+  const bool cores = dtype == LRS_BF16 && k % GK == 0 && lda % 8 == 0 && ((uintptr_t)a % 16) == 0 && ((uintptr_t)w % 16) == 0;
+  if (cores) {
+    dim3 grid(max_tiles, (n + GN - 1) / GN);
+    if (out_dtype == LRS_BF16)
+      moe_experts_bf16_kernel<bf16><<<grid, 256, 0, s>>>((bf16*)out, ldc, (const bf16*)a, lda, (const bf16*)w, n, k, sorted, tile_expert, top, gather, act);
+    else if (out_dtype == LRS_F32)
+      moe_experts_bf16_kernel<float><<<grid, 256, 0, s>>>((float*)out, ldc, (const bf16*)a, lda, (const bf16*)w, n, k, sorted, tile_expert, top, gather, act);
+    else
+      return lrs_fail("moe_experts: unknown output dtype %d", out_dtype);
+    return lrs_check_launch("moe_experts");
+  }
+  dim3 grid(max_tiles, (n + 63) / 64);
+#define RUN(T, TO) moe_experts_kernel<T, TO><<<grid, 256, 0, s>>>((TO*)out, ldc, (const T*)a, lda, (const T*)w, n, k, sorted, tile_expert, top, gather, act)
+  if (dtype == LRS_F32 && out_dtype == LRS_F32) RUN(float, float);
+  else if (dtype == LRS_BF16 && out_dtype == LRS_BF16) RUN(bf16, bf16);
+  else if (dtype == LRS_BF16 && out_dtype == LRS_F32) RUN(bf16, float);
+  else return lrs_fail("moe_experts: inputs of dtype %d with outputs of dtype %d are not served", dtype, out_dtype);
+#undef RUN
+  return lrs_check_launch("moe_experts");
+}
+
+// residual [tokens, hidden] += (norm of) sum_c weights[t, c] * rows[place[t, c]]; norm_w null: the plain sum.
+LRS_API int lrs_moe_combine(float* residual, const float* rows, int tokens, int hidden, const int* place, const float* weights,
+                            int top, const void* norm_w, int norm_dtype, float eps, void* stream) {
+  LRS_REQUIRE(tokens > 0 && hidden > 0 && top > 0, "moe_combine: bad sizes tokens=%d hidden=%d top=%d", tokens, hidden, top);
+  LRS_REQUIRE(!norm_w || eps > 0.f, "moe_combine: eps must be positive");
+  const size_t lds = (size_t)(hidden + 16) * sizeof(float);
+  LRS_REQUIRE(lds <= 64 * 1024, "moe_combine: a width of %d is too much", hidden);
+  hipStream_t s = (hipStream_t)stream;
+  if (norm_w && norm_dtype == LRS_BF16)
+    moe_combine_kernel<bf16><<<tokens, 256, lds, s>>>(residual, rows, hidden, place, weights, top, (const bf16*)norm_w, eps);
+  else
+    moe_combine_kernel<float><<<tokens, 256, lds, s>>>(residual, rows, hidden, place, weights, top, (const float*)norm_w, eps);
+  return lrs_check_launch("moe_combine");
+}

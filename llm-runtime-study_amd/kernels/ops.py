@@ -144,6 +144,18 @@ _SIGNATURES = {
     "lrs_choose_tokens_static_init": (c_int, []),
     "lrs_choose_tokens_static_max_parts": (c_int, []),
     "lrs_filter_logits": (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "lrs_round_rows": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_void_p]),
+    "lrs_norm_add": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_void_p]),
+    "lrs_delta_state_rows": (c_int, [c_int]),
+    "lrs_delta_rule": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
+                               c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p]),
+    "lrs_moe_tile_rows": (c_int, []),
+    "lrs_moe_max_tiles": (c_int, [c_int, c_int]),
+    "lrs_moe_route": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "lrs_moe_align": (c_int, [c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p]),
+    "lrs_moe_experts": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int,
+                                c_int, c_int, c_void_p]),
+    "lrs_moe_combine": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_float, c_void_p]),
 }
 
 
@@ -180,9 +192,10 @@ def library():
 # PLAN_OPS fixes the number of each entry point inside a plan; csrc/plan_dispatch.inc, made from this list
 # and _SIGNATURES by kernels/plan_codegen.py, is the other side (a test keeps the two in step).
 PLAN_OPS = ("lrs_add_into", "lrs_add_rmsnorm", "lrs_advance_decode", "lrs_advance_slots", "lrs_attention", "lrs_attention_decode",
-            "lrs_attention_prefill", "lrs_choose_tokens", "lrs_choose_tokens_split", "lrs_copy_to_pinned", "lrs_embed", "lrs_fill_i32",
+            "lrs_attention_prefill", "lrs_choose_tokens", "lrs_choose_tokens_split", "lrs_copy_to_pinned", "lrs_delta_rule", "lrs_embed", "lrs_fill_i32",
             "lrs_filter_logits", "lrs_gather_rows", "lrs_gemm", "lrs_gemm_lines_add_rmsnorm", "lrs_gemm_mid_add_norm_begin", "lrs_gemm_mid_qk_prep", "lrs_gemm_mid_scaled",
-            "lrs_gemm_norm_chain", "lrs_library_gemm", "lrs_qk_prep", "lrs_rmsnorm", "lrs_rope_table", "lrs_scale_rows", "lrs_silu_mul")
+            "lrs_gemm_norm_chain", "lrs_library_gemm", "lrs_moe_align", "lrs_moe_combine", "lrs_moe_experts", "lrs_moe_route", "lrs_norm_add",
+            "lrs_qk_prep", "lrs_rmsnorm", "lrs_rope_table", "lrs_round_rows", "lrs_scale_rows", "lrs_silu_mul")
 _PLAN_INDEX = {name: index for index, name in enumerate(PLAN_OPS)}
 
 
@@ -417,6 +430,21 @@ def add_rmsnorm(out: torch.Tensor, x: torch.Tensor, y: torch.Tensor, weight: tor
     _need(weight.is_contiguous() and weight.numel() == hidden, f"add_rmsnorm: weight must hold {hidden} values")
     _launch("lrs_add_rmsnorm", _dev(out, "out"), dtype_code(out.dtype), _dev(x, "x"), _dev(y, "y"), _dev(weight, "weight"),
                                      dtype_code(weight.dtype), n_rows, hidden, eps, _stream())
+
+
+def round_rows(out: torch.Tensor, x: torch.Tensor) -> None:
+    """out = the float32 rows x in out's dtype (the residual stream as the activation a sublayer reads)."""
+    _need(x.dtype == torch.float32 and x.is_contiguous() and out.is_contiguous() and out.shape == x.shape, "round_rows: out and x must be contiguous and of one shape")
+    _launch("lrs_round_rows", _dev(out, "out"), dtype_code(out.dtype), _dev(x, "x"), x.numel(), _stream())
+
+
+def norm_add(residual: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float) -> None:
+    """residual += weight * y * rsqrt(mean(y^2) + eps), row by row, in float32: the norm of a sublayer's output added to the stream."""
+    n_rows, hidden = y.shape
+    _need(residual.dtype == torch.float32 and y.dtype == torch.float32 and residual.is_contiguous() and y.is_contiguous()
+          and residual.shape[0] >= n_rows and residual.shape[1] == hidden, "norm_add: residual and y must be contiguous float32 [T, H]")
+    _need(weight.is_contiguous() and weight.numel() == hidden, f"norm_add: weight must hold {hidden} values")
+    _launch("lrs_norm_add", _dev(residual, "residual"), _dev(y, "y"), _dev(weight, "weight"), dtype_code(weight.dtype), n_rows, hidden, eps, _stream())
 
 
 def rope_table(cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor) -> None:
@@ -1095,3 +1123,103 @@ def filter_logits(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.
         _need(top_p.dtype == torch.float32 and top_p.numel() >= rows, "filter_logits: top_p must be float32 [R]")
     _launch("lrs_filter_logits", _dev(logits, "logits", torch.float32), stride, rows, vocab, _dev(temperature, "temperature"),
                                        None if top_k is None else _dev(top_k, "top_k"), None if top_p is None else _dev(top_p, "top_p"), _stream())
+
+
+# ------------------------------------------------------------------- gated delta rule
+def delta_state_floats(heads: int, kv_heads: int, dim: int, vdim: int, taps: int) -> int:
+    """Floats of one request's state row of a gated-delta-rule mixer: the matrix of every head in the order the scan
+    holds it (dim padded to a multiple of four), then the convolution's last taps - 1 inputs of every channel."""
+    rows = library().lrs_delta_state_rows(dim)
+    return heads * rows * 4 * vdim + (taps - 1) * (2 * kv_heads * dim + heads * vdim)
+
+
+def delta_rule(out: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, token_request: torch.Tensor, cu_seqlens: torch.Tensor,
+               slot_ids: torch.Tensor, requests: int, conv_weight: torch.Tensor, kv_heads: int, heads: int, dim: int, vdim: int,
+               a_log: torch.Tensor, dt_bias: torch.Tensor, norm_weight: torch.Tensor, eps: float, qkv: torch.Tensor, gates: torch.Tensor) -> None:
+    """One step of the gated delta rule for a ragged batch.  proj [T, >= C] holds each token's projections, columns
+    q (kv_heads*dim) | k (kv_heads*dim) | v (heads*vdim) | output gate (heads*vdim) | step size (heads) | decay input
+    (heads); state [slots, floats] float32 is read and written at the rows slot_ids names; out [T, heads*vdim]."""
+    tokens = out.shape[0]
+    channels = 2 * kv_heads * dim + heads * vdim
+    taps = conv_weight.shape[1]
+    _need(out.is_contiguous() and out.shape[1] == heads * vdim, "delta_rule: out must be contiguous [T, heads*vdim]")
+    _need(proj.shape[0] >= tokens and proj.shape[1] >= channels + heads * vdim + 2 * heads, "delta_rule: proj holds too few columns")
+    _need(state.dim() == 2 and state.dtype == torch.float32 and state.is_contiguous()
+          and state.shape[1] >= delta_state_floats(heads, kv_heads, dim, vdim, taps), "delta_rule: state rows are too short")
+    _need(conv_weight.shape == (channels, taps) and conv_weight.dtype == torch.float32 and conv_weight.is_contiguous(),
+          f"delta_rule: the convolution's weights must be float32 [{channels}, taps]")
+    for name, t, count in (("a_log", a_log, heads), ("dt_bias", dt_bias, heads), ("norm_weight", norm_weight, vdim)):
+        _need(t.dtype == torch.float32 and t.numel() == count and t.is_contiguous(), f"delta_rule: {name} must hold {count} float32 values")
+    for name, t, count in (("token_request", token_request, tokens), ("cu_seqlens", cu_seqlens, requests + 1), ("slot_ids", slot_ids, requests)):
+        _need(t.dtype == torch.int32 and t.numel() >= count and t.is_contiguous(), f"delta_rule: {name} must be int32 [{count}]")
+    _need(qkv.dtype == torch.float32 and qkv.is_contiguous() and qkv.numel() >= tokens * channels, "delta_rule: qkv scratch too small")
+    _need(gates.dtype == torch.float32 and gates.is_contiguous() and gates.numel() >= tokens * 2 * heads, "delta_rule: gates scratch too small")
+    _launch("lrs_delta_rule", _dev(out, "out"), dtype_code(out.dtype), _dev(proj, "proj"), dtype_code(proj.dtype), _rows(proj, "proj"), tokens,
+            requests, _dev(token_request, "token_request"), _dev(cu_seqlens, "cu_seqlens"), _dev(slot_ids, "slot_ids"), _dev(state, "state"),
+            state.stride(0), _dev(conv_weight, "conv_weight"), taps, kv_heads, heads, dim, vdim, _dev(a_log, "a_log"), _dev(dt_bias, "dt_bias"),
+            _dev(norm_weight, "norm_weight"), eps, _dev(qkv, "qkv"), _dev(gates, "gates"), _stream())
+
+
+# ------------------------------------------------------------------- routed experts
+@functools.lru_cache(maxsize=1)
+def moe_tile_rows() -> int:
+    return library().lrs_moe_tile_rows()
+
+
+def moe_max_tiles(pairs: int, experts: int) -> int:
+    """The most row tiles that `pairs` (token, choice) pairs of `experts` experts fill once sorted by expert."""
+    return min(pairs, pairs // moe_tile_rows() + experts)
+
+
+def moe_route(logits: torch.Tensor, bias: torch.Tensor | None, ids: torch.Tensor, weights: torch.Tensor) -> None:
+    """ids, weights [T, top]: per token the `top` largest of logits [T, E] (+ bias) and the softmax over those alone."""
+    tokens, top = ids.shape
+    experts = logits.shape[1]
+    _need(logits.dtype == torch.float32 and logits.shape[0] >= tokens and logits.stride(1) == 1, "moe_route: logits must be float32 [T, E]")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == experts and bias.is_contiguous()), "moe_route: bias must hold E float32 values")
+    _need(ids.dtype == torch.int32 and ids.is_contiguous() and weights.dtype == torch.float32 and weights.is_contiguous()
+          and weights.shape == ids.shape, "moe_route: ids must be int32 [T, top] and weights float32 [T, top]")
+    _launch("lrs_moe_route", _dev(logits, "logits"), logits.stride(0), None if bias is None else _dev(bias, "bias"), _dev(ids, "ids"),
+            _dev(weights, "weights"), tokens, experts, top, _stream())
+
+
+def moe_align(ids: torch.Tensor, experts: int, sorted_pairs: torch.Tensor, place: torch.Tensor, tile_expert: torch.Tensor) -> None:
+    """Sorts the (token, choice) pairs of ids [T, top] by expert: sorted_pairs [tiles * tile rows] (pair index, -1 in the
+    rows that pad an expert's run), place [T * top] (the row of each pair), tile_expert [tiles] (-1: tile not in use)."""
+    pairs, tiles = ids.numel(), tile_expert.numel()
+    for name, t in (("ids", ids), ("sorted_pairs", sorted_pairs), ("place", place), ("tile_expert", tile_expert)):
+        _need(t.dtype == torch.int32 and t.is_contiguous(), f"moe_align: {name} must be contiguous int32")
+    _need(tiles >= moe_max_tiles(pairs, experts) and sorted_pairs.numel() >= tiles * moe_tile_rows() and place.numel() >= pairs,
+          "moe_align: the lists are too short for the step")
+    _launch("lrs_moe_align", _dev(ids, "ids"), pairs, experts, _dev(sorted_pairs, "sorted_pairs"), sorted_pairs.numel(), _dev(place, "place"),
+            _dev(tile_expert, "tile_expert"), tiles, _stream())
+
+
+def moe_experts(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, sorted_pairs: torch.Tensor, tile_expert: torch.Tensor, top: int,
+                gather: bool, relu_squared: bool) -> None:
+    """out [tiles * tile rows, N] = rows of `a` times w[expert of the tile] [N, K], transposed, for every tile in use.
+    gather: the row of a sorted pair is a[pair // top] (tokens); else `a` is in sorted order itself."""
+    experts, n, k = w.shape
+    tiles = tile_expert.numel()
+    _need(w.is_contiguous() and a.dtype == w.dtype and a.shape[1] == k, "moe_experts: a [*, K] and w [E, N, K] must agree")
+    _need(out.shape == (tiles * moe_tile_rows(), n) and out.dtype in (w.dtype, torch.float32), "moe_experts: out must be [tiles * tile rows, N]")
+    _need(gather or a.shape[0] >= tiles * moe_tile_rows(), "moe_experts: sorted rows missing")
+    _need(sorted_pairs.numel() >= tiles * moe_tile_rows(), "moe_experts: sorted list too short")
+    _launch("lrs_moe_experts", _dev(out, "out"), dtype_code(out.dtype), _rows(out, "out"), _dev(a, "a"), _dev(w, "w"), dtype_code(w.dtype),
+            _rows(a, "a"), n, k, _dev(sorted_pairs, "sorted_pairs", torch.int32), _dev(tile_expert, "tile_expert", torch.int32), tiles, top,
+            int(gather), int(relu_squared), _stream())
+
+
+def moe_combine(residual: torch.Tensor, rows: torch.Tensor, place: torch.Tensor, weights: torch.Tensor, norm_weight: torch.Tensor | None,
+                eps: float = 0.0) -> None:
+    """residual [T, H] += sum over a token's choices of weights[t, c] * rows[place[t, c]]; with norm_weight: the RMS
+    norm (weight norm_weight, eps) of that sum instead of the sum itself."""
+    tokens, top = weights.shape
+    hidden = rows.shape[1]
+    _need(residual.dtype == torch.float32 and residual.is_contiguous() and residual.shape[0] >= tokens and residual.shape[1] == hidden
+          and rows.dtype == torch.float32 and rows.is_contiguous(), "moe_combine: residual [T, H] and rows [*, H] must be contiguous float32")
+    _need(place.dtype == torch.int32 and place.numel() >= tokens * top and place.is_contiguous() and weights.dtype == torch.float32
+          and weights.is_contiguous(), "moe_combine: place must be int32 [T * top] and weights float32 [T, top]")
+    _need(norm_weight is None or (norm_weight.numel() == hidden and norm_weight.is_contiguous()), "moe_combine: norm weight must hold H values")
+    _launch("lrs_moe_combine", _dev(residual, "residual"), _dev(rows, "rows"), tokens, hidden, _dev(place, "place"), _dev(weights, "weights"), top,
+            None if norm_weight is None else _dev(norm_weight, "norm_weight"), 0 if norm_weight is None else dtype_code(norm_weight.dtype), eps, _stream())

@@ -12,7 +12,7 @@ import torch
 
 from ..kernels import ops
 from ..parts import TensorSpec, create
-from ..parts.base import flops_of, under
+from ..parts.base import Renamed, flops_of, under
 from ..parts.linear import linear
 from .spec import ModelSpec
 
@@ -41,12 +41,16 @@ class DecoderModel:
         for part, prefix in self._around():
             out.update({f"{prefix}.{name}": t for name, t in part.tensors().items()})
         out[spec.head_name] = TensorSpec((spec.vocab_size, spec.hidden_size), role="matrix", optional=spec.tie_head)
+        if spec.checkpoint_name is not None:
+            out = {spec.checkpoint_name(name): t for name, t in out.items()}
         return out
 
     def bind(self, weights: dict[str, torch.Tensor], dtype: torch.dtype) -> None:
         """Hand every part its tensors; `dtype` is the activation (and matrix) dtype of the run."""
         spec = self.spec
         self.dtype = dtype
+        if spec.checkpoint_name is not None:
+            weights = Renamed(weights, spec.checkpoint_name)
         self.embedding = weights[spec.embedding_name].to(dtype).contiguous()
         head = weights.get(spec.head_name)
         self.head = self.embedding if head is None else head.to(dtype).contiguous()

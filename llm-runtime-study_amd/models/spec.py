@@ -12,11 +12,15 @@ An architecture turns its typed configuration into a ModelSpec; everything after
             stream right after the embedding (a learned or absolute position signal, a scale)
             and on the float32 logits (a scale, a soft cap); their tensors are named
             `<after_embedding_prefix>.<name>` and `<after_head_prefix>.<name>`.
+  checkpoint_name
+            for checkpoints that name their tensors otherwise than the parts do: the function from a part's
+            full tensor name to the checkpoint's.
 """
 
 from __future__ import annotations
 
 from dataclasses import dataclass, field
+from typing import Callable
 
 from ..parts import PartSpec
 
@@ -49,6 +53,8 @@ class ModelSpec:
     after_head: PartSpec | None = None
     after_embedding_prefix: str = "model.after_embedding"
     after_head_prefix: str = "after_head"
+    # the checkpoint's name of a tensor, given the name the parts make for it (prefixes and all); None: the same
+    checkpoint_name: Callable[[str], str] | None = field(default=None, compare=False)
     extra: dict = field(default_factory=dict, compare=False)
 
     def validate(self) -> None:

@@ -9,7 +9,11 @@ h // (nq/nkv) for query head h (18-33), then the output projection without bias.
 
 q, k and v come from one stacked [nq*d + 2*nkv*d, H] product.  When `kv_shared` is set the
 layer owns no keys or values: it projects queries only and attends to the cache of the layer
-it is told to read.  `window` keeps keys with p - window < j <= p.
+it is told to read.  `window` keeps keys with p - window < j <= p.  With `values_from_keys` there is no
+value projection: a position's value is its key as projected, before the per-head norm and the rotation; the
+key matrix is stacked a second time where the value matrix would be, so that every kernel after the product sees
+the usual row of q, k and v heads (the product makes those columns twice, from the same weights and inputs).
+`forward(..., accumulate=False)` stores the output projection into the float32 rows it is given instead of adding to them.
 """
 
 from __future__ import annotations
@@ -29,11 +33,12 @@ class GQAAttention(Part):
     takes_lazy_norm = True
     begins_next_norm = True
     wants_query_groups = True   # ragged steps go to a kernel that walks groups of a request's consecutive tokens
+    can_overwrite = True        # forward(..., accumulate=False) stores its output
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, *,
                  position: PartSpec = PartSpec("none"), qk_norm: bool = False, qk_norm_eps: float = 1e-6,
                  bias: bool = False, scale: float | None = None, window: int | None = None,
-                 kv_shared: bool = False):
+                 kv_shared: bool = False, values_from_keys: bool = False):
         for name, value in (("hidden_size", hidden_size), ("num_heads", num_heads), ("num_kv_heads", num_kv_heads), ("head_dim", head_dim)):
             if value <= 0:
                 raise ValueError(f"{name} must be positive, got {value}")
@@ -49,13 +54,15 @@ class GQAAttention(Part):
         self.position = create("position", position)
         self.qk_norm, self.qk_norm_eps, self.bias = qk_norm, qk_norm_eps, bias
         self.scale = 1.0 / math.sqrt(head_dim) if scale is None else scale
-        self.window, self.kv_shared = window, kv_shared
+        if values_from_keys and kv_shared:
+            raise ValueError("a layer that owns no keys has no values to take from them")
+        self.window, self.kv_shared, self.values_from_keys = window, kv_shared, values_from_keys
         self.w_qkv = self.b_qkv = self.w_o = self.q_norm = self.k_norm = None
 
     # ------------------------------------------------------------------ weights
     def tensors(self):
         h, d = self.hidden_size, self.head_dim
-        names = ("q_proj",) if self.kv_shared else ("q_proj", "k_proj", "v_proj")
+        names = ("q_proj",) if self.kv_shared else ("q_proj", "k_proj") if self.values_from_keys else ("q_proj", "k_proj", "v_proj")
         widths = {"q_proj": self.num_heads * d, "k_proj": self.num_kv_heads * d, "v_proj": self.num_kv_heads * d}
         specs = {f"{n}.weight": TensorSpec((widths[n], h)) for n in names}
         if self.bias:
@@ -68,7 +75,7 @@ class GQAAttention(Part):
         return specs
 
     def bind(self, weights, dtype):
-        names = ("q_proj",) if self.kv_shared else ("q_proj", "k_proj", "v_proj")
+        names = ("q_proj",) if self.kv_shared else ("q_proj", "k_proj", "k_proj") if self.values_from_keys else ("q_proj", "k_proj", "v_proj")
         self.w_qkv = torch.cat([weights[f"{n}.weight"] for n in names], 0).to(dtype).contiguous()
         self.b_qkv = torch.cat([weights[f"{n}.bias"] for n in names], 0).to(dtype).contiguous() if self.bias else None
         self.w_o = weights["o_proj.weight"].to(dtype).contiguous()
@@ -150,7 +157,7 @@ class GQAAttention(Part):
     PREPARE_INSIDE_ROWS = 16     # rows of a decode step up to which the attention kernel prepares q, k and v itself
 
     # ------------------------------------------------------------------ forward
-    def forward(self, ctx, x, residual, cache, then_norm=None):
+    def forward(self, ctx, x, residual, cache, then_norm=None, accumulate: bool = True):
         if cache is None:
             raise ValueError("attention needs a paged cache (its own, or the one it is told to read)")
         t, d, nq = rows_of(x), self.head_dim, self.num_heads
@@ -249,7 +256,7 @@ class GQAAttention(Part):
         else:
             ops.attention(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_slot, ctx.positions,
                           nq, self.scale, self.window or 0)
-        return linear(ctx, residual, out, self.w_o, accumulate=True, then_norm=then_norm)
+        return linear(ctx, residual, out, self.w_o, accumulate=accumulate, then_norm=then_norm)
 
 
 register("mixer", "gqa_attention", GQAAttention)

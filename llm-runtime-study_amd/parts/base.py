@@ -129,6 +129,26 @@ class Under(MappingView):
         return isinstance(name, str) and self._prefix + name in self._weights
 
 
+class Renamed(MappingView):
+    """`weights` looked up under other names: asking for `name` gives weights[rename(name)].  For checkpoints that
+    name their tensors otherwise than the parts do.  Lookups only: it cannot list its names."""
+
+    def __init__(self, weights: Mapping[str, torch.Tensor], rename: Callable[[str], str]):
+        self._weights, self._rename = weights, rename
+
+    def __getitem__(self, name: str) -> torch.Tensor:
+        return self._weights[self._rename(name)]
+
+    def __contains__(self, name) -> bool:
+        return isinstance(name, str) and self._rename(name) in self._weights
+
+    def __iter__(self):
+        raise TypeError("renamed tensors are looked up by name, not listed")
+
+    def __len__(self) -> int:
+        return len(self._weights)
+
+
 def under(weights: Mapping[str, torch.Tensor], prefix: str) -> Mapping[str, torch.Tensor]:
     """What a part that owns the names under `prefix` is given to bind()."""
     return Under(weights, prefix)

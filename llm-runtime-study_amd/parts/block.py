@@ -3,10 +3,20 @@
 PreNormBlock (reference mini_llm/model/qwen.py:58-72):
     h = h + mixer(norm1(h));  h = h + feed_forward(norm2(h))
 The two sums happen inside the parts, which add into the float32 residual stream.
+
+OutputNormBlock: the sublayers read the stream itself and the norms are applied to what they give out:
+    h = h + norm1(mixer(h));  h = h + norm2(feed_forward(h))      (the feed-forward may be absent)
+A sublayer writes its output into a float32 buffer of the step (a part that says `can_overwrite` stores it, any
+other adds into the buffer after it has been cleared), and the norm adds the normalised rows into the stream; a
+feed-forward that says `applies_output_norm` is given the norm and does both itself, in the kernel that sums up
+its output.
 """
 
 from __future__ import annotations
 
+import torch
+
+from ..kernels import ops
 from .base import Part, PartSpec, create, flops_of, register, under
 from .linear import materialize
 
@@ -87,3 +97,87 @@ class PreNormBlock(Part):
 
 
 register("block", "prenorm", PreNormBlock)
+
+
+class OutputNormBlock(Part):
+    def __init__(self, mixer: PartSpec, mixer_norm: PartSpec, feed_forward: PartSpec | None = None, ff_norm: PartSpec | None = None,
+                 names: dict | None = None):
+        if (feed_forward is None) != (ff_norm is None):
+            raise ValueError("a feed-forward and its norm come together")
+        self.mixer = create("mixer", mixer)
+        self.mixer_norm = create("norm", mixer_norm)
+        self.feed_forward = None if feed_forward is None else create("feed_forward", feed_forward)
+        self.ff_norm = None if ff_norm is None else create("norm", ff_norm)
+        for norm in (self.mixer_norm, self.ff_norm):
+            if norm is not None and not callable(getattr(norm, "add_normed", None)):
+                raise ValueError("a norm of a sublayer's output must offer add_normed(ctx, residual, y)")
+        self.names = {"mixer": "mixer", "feed_forward": "feed_forward", "mixer_norm": "mixer_norm", "ff_norm": "ff_norm"}
+        self.names.update(names or {})
+
+    def _children(self):
+        return [(self.names[k], getattr(self, k)) for k in ("mixer_norm", "mixer", "ff_norm", "feed_forward") if getattr(self, k) is not None]
+
+    def tensors(self):
+        return {f"{prefix}.{name}": spec for prefix, part in self._children() for name, spec in part.tensors().items()}
+
+    def bind(self, weights, dtype):
+        for prefix, part in self._children():
+            part.bind(under(weights, prefix + "."), dtype)
+
+    def weight_bytes(self):
+        return sum(part.weight_bytes() for _, part in self._children())
+
+    def flops(self, tokens, pairs):
+        return sum(flops_of(part, tokens, pairs) for _, part in self._children())
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(part, "graph_safe", False) for _, part in self._children())
+
+    @property
+    def plan_safe(self) -> bool:
+        return all(getattr(part, "plan_safe", False) for _, part in self._children())
+
+    @property
+    def wants_query_groups(self) -> bool:
+        return getattr(self.mixer, "wants_query_groups", False)
+
+    @staticmethod
+    def _input(ctx, h):
+        """The stream as the activation a sublayer reads: itself in float32 runs, else rounded once."""
+        if ctx.dtype == torch.float32:
+            return h
+        x = ctx.scratch("stream_rounded", tuple(h.shape), ctx.dtype)
+        ops.round_rows(x, h)
+        return x
+
+    @staticmethod
+    def _cleared(ctx, h):
+        y = ctx.scratch("sublayer_out", tuple(h.shape), torch.float32)
+        ops.fill_i32(y.view(torch.int32), 0)
+        return y
+
+    def forward(self, ctx, h, cache):
+        x = self._input(ctx, h)
+        if getattr(self.mixer, "can_overwrite", False):
+            y = ctx.scratch("sublayer_out", tuple(h.shape), torch.float32)
+            self.mixer.forward(ctx, x, y, cache, accumulate=False)
+        else:
+            y = self._cleared(ctx, h)
+            self.mixer.forward(ctx, x, y, cache)
+        self.mixer_norm.add_normed(ctx, h, y)
+        if self.feed_forward is None:
+            return
+        x = self._input(ctx, h)
+        if getattr(self.feed_forward, "applies_output_norm", False) and getattr(self.ff_norm, "rms_parameters", None) is not None:
+            self.feed_forward.forward(ctx, x, h, output_norm=self.ff_norm)
+            return
+        y = self._cleared(ctx, h)
+        self.feed_forward.forward(ctx, x, y)
+        self.ff_norm.add_normed(ctx, h, y)
+
+
+register("block", "outnorm", OutputNormBlock)

@@ -1,0 +1,107 @@
+"""Gated delta rule: a mixer whose memory is one matrix per head, updated token by token.
+
+For a token with input x, per head h (key group h // (heads / kv_heads), as in grouped-query attention):
+    q, k  = unit(silu(conv(W_q x))), unit(silu(conv(W_k x)))        q also times head_dim ** -0.5
+    v     = silu(conv(W_v x))
+    beta  = sigmoid(W_b x)                                           the step size
+    g     = exp(-exp(A_log) * softplus(W_a x + dt_bias))             the decay
+    S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q     S [head_dim, value_dim], zero at a sequence's start
+    out   = W_o (rms_norm(o) * norm_weight * silu(W_g x))            the norm per head over value_dim
+`conv` is a causal convolution over time, a few taps per channel, no bias, zeros before the sequence's start;
+`unit(z) = z / sqrt(sum(z^2) + 1e-6)`.  The gates, the unit norms, the state and the read-out are float32 in
+every run; the projections that feed them are written in float32 too.
+
+All six input projections are one stacked product.  What a request keeps between steps is one float32 row: the
+matrices of all heads, then the convolution's last taps - 1 inputs of every channel (`StateNeed`); the cache
+manager hands out the rows, clears a row at admission and the kernels find a request's row by its slot.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from .base import Part, StateNeed, TensorSpec, register
+from .linear import linear, materialize, rows_of
+
+STATE_LANES = 4      # lanes that share a column of a head's matrix in the scan kernel; head_dim is padded to a multiple of it
+
+
+class GatedDeltaRule(Part):
+    graph_safe = True   # launches only this package's kernels on arena buffers, reads the step's data on the device
+    plan_safe = True
+    can_overwrite = True
+
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, conv_taps: int, norm_eps: float):
+        for name, value in (("hidden_size", hidden_size), ("num_heads", num_heads), ("num_kv_heads", num_kv_heads), ("head_dim", head_dim),
+                            ("value_dim", value_dim), ("conv_taps", conv_taps)):
+            if value <= 0:
+                raise ValueError(f"{name} must be positive, got {value}")
+        if num_heads % num_kv_heads != 0:
+            raise ValueError(f"num_heads must be divisible by num_kv_heads, got {num_heads} and {num_kv_heads}")
+        if head_dim > 256 or value_dim > 256:
+            raise ValueError(f"the scan kernel takes head_dim and value_dim up to 256, got {head_dim} and {value_dim}")
+        if norm_eps <= 0:
+            raise ValueError(f"norm_eps must be positive, got {norm_eps}")
+        self.hidden_size, self.num_heads, self.num_kv_heads = hidden_size, num_heads, num_kv_heads
+        self.head_dim, self.value_dim, self.conv_taps, self.norm_eps = head_dim, value_dim, conv_taps, norm_eps
+        self.channels = 2 * num_kv_heads * head_dim + num_heads * value_dim          # what passes the convolution: q, k, v
+        self.columns = self.channels + num_heads * value_dim + 2 * num_heads          # ... and the output gate, step size, decay input
+        self.w_in = self.w_o = self.conv = self.a_log = self.dt_bias = self.norm = None
+
+    def _projections(self):
+        qk, v = self.num_kv_heads * self.head_dim, self.num_heads * self.value_dim
+        return (("q_proj", qk), ("k_proj", qk), ("v_proj", v), ("g_proj", v), ("b_proj", self.num_heads), ("a_proj", self.num_heads))
+
+    def tensors(self):
+        specs = {f"{name}.weight": TensorSpec((width, self.hidden_size)) for name, width in self._projections()}
+        for name, width in self._projections()[:3]:
+            specs[f"{name[0]}_conv.weight"] = TensorSpec((width, self.conv_taps))
+        specs["A_log"] = TensorSpec((self.num_heads,), role="bias")
+        specs["dt_bias"] = TensorSpec((self.num_heads,), role="bias")
+        specs["norm.weight"] = TensorSpec((self.value_dim,), role="norm")
+        specs["o_proj.weight"] = TensorSpec((self.hidden_size, self.num_heads * self.value_dim))
+        return specs
+
+    def bind(self, weights, dtype):
+        stacked = torch.cat([weights[f"{name}.weight"] for name, _ in self._projections()], 0).to(dtype)
+        pad = -stacked.shape[0] % 16          # whole groups of 16 output columns suit every product kernel
+        if pad:
+            stacked = torch.cat((stacked, stacked.new_zeros(pad, self.hidden_size)), 0)
+        self.w_in = stacked.contiguous()
+        self.conv = torch.cat([weights[f"{name}_conv.weight"] for name in "qkv"], 0).float().contiguous()
+        self.a_log, self.dt_bias = weights["A_log"].float().contiguous(), weights["dt_bias"].float().contiguous()
+        self.norm = weights["norm.weight"].float().contiguous()
+        self.w_o = weights["o_proj.weight"].to(dtype).contiguous()
+
+    def weight_bytes(self):
+        return (self.w_in.numel() + self.w_o.numel()) * self.w_o.element_size()
+
+    def flops(self, tokens, pairs):
+        # the projections, and per token and head the two products with the state and its update
+        return super().flops(tokens, pairs) + 6.0 * tokens * self.num_heads * self.head_dim * self.value_dim
+
+    def state_floats(self) -> int:
+        rows = -(-self.head_dim // STATE_LANES)
+        return self.num_heads * rows * STATE_LANES * self.value_dim + (self.conv_taps - 1) * self.channels
+
+    def cache_need(self):
+        return StateNeed((self.state_floats(),), torch.float32)
+
+    def forward(self, ctx, x, residual, cache, then_norm=None, accumulate: bool = True):
+        if cache is None or cache.state is None:
+            raise ValueError("the gated delta rule needs a state row per request")
+        t = rows_of(x)
+        x = materialize(ctx, x)
+        proj = ctx.scratch("delta_proj", (t, self.w_in.shape[0]), torch.float32)
+        linear(ctx, proj, x, self.w_in)
+        out = ctx.scratch("delta_out", (t, self.num_heads * self.value_dim), ctx.dtype)
+        qkv = ctx.scratch("delta_qkv", (t, self.channels), torch.float32)
+        gates = ctx.scratch("delta_gates", (t, 2 * self.num_heads), torch.float32)
+        ops.delta_rule(out, proj, cache.state, ctx.token_request, ctx.cu_seqlens_q, ctx.slot_ids, ctx.R, self.conv, self.num_kv_heads,
+                       self.num_heads, self.head_dim, self.value_dim, self.a_log, self.dt_bias, self.norm, self.norm_eps, qkv, gates)
+        linear(ctx, residual, out, self.w_o, accumulate=accumulate)
+        return None
+
+
+register("mixer", "gated_delta_rule", GatedDeltaRule)

@@ -1,0 +1,99 @@
+"""Routed experts: a feed-forward made of many small ones, of which every token runs a few.
+
+    z = W_router x (+ bias)                        float32 (x may be the activation's rounding)
+    chosen = the `top` largest z;  p = softmax(z[chosen])
+    out = sum over chosen e of p_e * W_down_e act(W_up_e x)         act: the square of relu, or relu
+
+On the device: the router product, the choice per token, one sort of the step's (token, choice) pairs by expert
+into runs padded to whole row tiles, two grouped products over the sorted rows (the activation in the first one's
+epilogue), and one kernel that adds a token's rows up in the order of its choices, which can also apply the norm
+of a layer that normalises outputs and add the result into the stream (`applies_output_norm`).  Nothing is read
+on the host: the launches are sized by the step's shape alone (at most pairs / tile + experts tiles).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from .base import Part, TensorSpec, register
+from .linear import kernels_of, materialize, rows_of, workspace_of
+
+ACTIVATIONS = ("relu_squared",)
+
+
+class RoutedExperts(Part):
+    graph_safe = True
+    plan_safe = True
+    applies_output_norm = True    # forward(..., output_norm=norm): residual += norm(out) instead of residual += out
+
+    def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int, top: int, router_bias: bool = False,
+                 activation: str = "relu_squared"):
+        if min(hidden_size, intermediate_size, num_experts, top) <= 0:
+            raise ValueError("hidden_size, intermediate_size, num_experts and top must be positive")
+        if top > num_experts:
+            raise ValueError(f"a token cannot run {top} of {num_experts} experts")
+        if num_experts > 512:
+            raise ValueError(f"the routing kernel takes up to 512 experts, got {num_experts}")
+        if activation not in ACTIVATIONS:
+            raise ValueError(f"unknown activation {activation!r}; known: {', '.join(ACTIVATIONS)}")
+        self.hidden_size, self.intermediate_size, self.num_experts, self.top = hidden_size, intermediate_size, num_experts, top
+        self.router_bias, self.activation = router_bias, activation
+        self.router = self.bias = self.up = self.down = None
+
+    def tensors(self):
+        h, i = self.hidden_size, self.intermediate_size
+        specs = {"router.weight": TensorSpec((self.num_experts, h))}
+        if self.router_bias:
+            specs["router.bias"] = TensorSpec((self.num_experts,), role="bias")
+        for e in range(self.num_experts):
+            specs[f"experts.{e}.up.weight"] = TensorSpec((i, h))
+            specs[f"experts.{e}.down.weight"] = TensorSpec((h, i))
+        return specs
+
+    def bind(self, weights, dtype):
+        router = weights["router.weight"].to(dtype)
+        pad = -router.shape[0] % 16           # whole groups of 16 output columns suit every product kernel
+        if pad:
+            router = torch.cat((router, router.new_zeros(pad, self.hidden_size)), 0)
+        self.router = router.contiguous()
+        self.bias = weights["router.bias"].float().contiguous() if self.router_bias else None
+        self.up = torch.stack([weights[f"experts.{e}.up.weight"].to(dtype) for e in range(self.num_experts)]).contiguous()
+        self.down = torch.stack([weights[f"experts.{e}.down.weight"].to(dtype) for e in range(self.num_experts)]).contiguous()
+
+    def weight_bytes(self):
+        """What a decode step of one token reads: the router and the chosen experts."""
+        chosen = 2 * self.top * self.hidden_size * self.intermediate_size
+        return (self.router.numel() + chosen) * self.up.element_size()
+
+    def flops(self, tokens, pairs):
+        return 2.0 * tokens * (self.num_experts * self.hidden_size + 2 * self.top * self.hidden_size * self.intermediate_size)
+
+    def forward(self, ctx, x, residual, then_norm=None, output_norm=None):
+        t = rows_of(x)
+        x = materialize(ctx, x)
+        experts, top = self.num_experts, self.top
+        logits = ctx.scratch("moe_logits", (t, self.router.shape[0]), torch.float32)
+        ops.gemm(logits, x, self.router, choice=kernels_of(ctx), workspace=workspace_of(ctx) if ctx.dtype == torch.bfloat16 else None)
+        ids = ctx.scratch("moe_ids", (t, top), torch.int32)
+        weights = ctx.scratch("moe_weights", (t, top), torch.float32)
+        ops.moe_route(logits[:, :experts], self.bias, ids, weights)
+        tiles = ops.moe_max_tiles(t * top, experts)
+        rows = tiles * ops.moe_tile_rows()
+        sorted_pairs = ctx.scratch("moe_sorted", (rows,), torch.int32)
+        place = ctx.scratch("moe_place", (t * top,), torch.int32)
+        tile_expert = ctx.scratch("moe_tile_expert", (tiles,), torch.int32)
+        ops.moe_align(ids, experts, sorted_pairs, place, tile_expert)
+        hidden = ctx.scratch("moe_hidden", (rows, self.intermediate_size), ctx.dtype)
+        ops.moe_experts(hidden, x, self.up, sorted_pairs, tile_expert, top, gather=True, relu_squared=True)
+        outputs = ctx.scratch("moe_outputs", (rows, self.hidden_size), torch.float32)
+        ops.moe_experts(outputs, hidden, self.down, sorted_pairs, tile_expert, top, gather=False, relu_squared=False)
+        if output_norm is None:
+            ops.moe_combine(residual, outputs, place, weights, None)
+        else:
+            weight, eps = output_norm.rms_parameters()
+            ops.moe_combine(residual, outputs, place, weights, weight, eps)
+        return None
+
+
+register("feed_forward", "routed_experts", RoutedExperts)

@@ -2,6 +2,13 @@
 
 Formula (reference mini_llm/nn/norm.py:42-46): y = w * x * rsqrt(mean(x^2) + eps), statistics
 in float32.  The kernel rounds once, at the output, to the activation dtype.
+
+`unit_offset`: the checkpoint stores the weight around zero and the norm multiplies by 1 + w; the sum is made
+once, in float32, when the weights are bound, so every kernel sees a plain weight.
+
+Besides `forward` (the norm of the stream, for a sublayer to read) a norm can be applied to what a sublayer gives
+out: `add_normed(ctx, residual, y)` adds the norm of the float32 rows `y` into the stream, for layer arrangements
+that normalise outputs (parts/block.py, OutputNormBlock).
 """
 
 from __future__ import annotations
@@ -16,19 +23,25 @@ class RMSNorm(Part):
     plan_safe = True
     has_lazy_form = True
 
-    def __init__(self, size: int, eps: float):
+    def __init__(self, size: int, eps: float, unit_offset: bool = False):
         if size <= 0:
             raise ValueError(f"size must be positive, got {size}")
         if eps <= 0:
             raise ValueError(f"eps must be positive, got {eps}")
-        self.size, self.eps = size, eps
+        self.size, self.eps, self.unit_offset = size, eps, unit_offset
         self.weight = None
 
     def tensors(self):
-        return {"weight": TensorSpec((self.size,), role="norm")}
+        return {"weight": TensorSpec((self.size,), role="bias" if self.unit_offset else "norm")}
 
     def bind(self, weights, dtype):
         self.weight = weights["weight"]
+        if self.unit_offset:
+            self.weight = (1.0 + self.weight.float()).contiguous()
+
+    def add_normed(self, ctx, residual, y):
+        """residual += this norm of the float32 rows y (what a sublayer gave out)."""
+        ops.norm_add(residual, y, self.weight, self.eps)
 
     def rms_parameters(self):
         """(weight, eps): says that this norm is w * x * rsqrt(mean(x^2) + eps), so that the matrix
