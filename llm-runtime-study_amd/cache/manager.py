@@ -173,10 +173,10 @@ class CacheManager:
         return len(self._free_slots)
 
     def free_pages(self, group: int = 0) -> int:
-        return self.groups[group].pool.free_pages
+        return self.groups[group].pool.free_pages if self.groups else 0     # a model of state mixers alone keeps no pages
 
     def used_pages(self, group: int = 0) -> int:
-        return self.groups[group].pool.used_pages
+        return self.groups[group].pool.used_pages if self.groups else 0
 
     @property
     def used_tokens(self) -> int:
@@ -378,6 +378,8 @@ class CacheManager:
 
     def tables_match_device(self) -> bool:
         """Whether the device's block tables equal the host's in every entry that is not waiting in table_patches()."""
+        if self.device_tables is None:       # no paged group, or no storage: nothing to differ
+            return True
         expected = self._tables_host.copy()
         got = self.device_tables.cpu().numpy().copy()
         for g, slot, first, end in self._dirty:

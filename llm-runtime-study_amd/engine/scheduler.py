@@ -185,7 +185,7 @@ class BatchScheduler:
             entries, rows = self._build_batch()
             if entries:
                 started = self._now()
-                logits = self.runner.step(entries)
+                logits = self.runner.step(entries, keep_states=False)        # a failure gives every request up (abort_all)
                 tokens = self.sampler.choose(logits, [row for _, row in rows]) if rows else []
                 # reading the tokens has waited for the step; a step that samples nothing stays in flight
                 seconds = self._now(wait=False) - started if started is not None and rows else None
@@ -331,9 +331,9 @@ class BatchScheduler:
         entries = [StepEntry(r.cache, [r.next_token], [0]) for r in running]
         started = self._now()
         if getattr(self.runner, "decode_steps_sample", False):
-            chosen = self.runner.decode_steps(entries, steps, [SamplingRow(r.sampling, r.seed, r.produced) for r in running])
+            chosen = self.runner.decode_steps(entries, steps, [SamplingRow(r.sampling, r.seed, r.produced) for r in running], keep_states=False)
         else:
-            chosen = self.runner.decode_steps(entries, steps)
+            chosen = self.runner.decode_steps(entries, steps, keep_states=False)
         seconds = (self._now(wait=False) - started) / steps if started is not None else None     # the tokens are back: the launch has finished
         alive = running
         for tokens in chosen:

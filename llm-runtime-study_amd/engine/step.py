@@ -520,15 +520,18 @@ class ModelRunner:
         (ctx.token_ids, ctx.positions, ctx.token_request, ctx.token_slot, ctx.logit_rows, ctx.cu_seqlens_q, ctx.seq_lens_k, ctx.slot_ids,
          ctx.qblock_token0, ctx.qblock_count, ctx.counts, ctx._groups) = views
 
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor | None:
+    def step(self, entries: Sequence[StepEntry], keep_states: bool = True) -> torch.Tensor | None:
         """Run one step; returns float32 logits [wanted, vocab] on the device, or None if none is wanted.
 
-        The logits lie in a buffer that the next step writes again: read or copy them before it."""
+        The logits lie in a buffer that the next step writes again: read or copy them before it.
+        keep_states: copies of the requests' state rows are kept during the step and put back if it fails (for a mixer
+        whose state is a matrix per head that is megabytes a request and layer); a caller that gives its requests up
+        after a failure anyway, as the scheduler does, says False and saves the copy."""
         self.validate(entries)
         self._follow_construction()
         before = [entry.cache.length for entry in entries]
         extended = []
-        states = self.cache.snapshot_state([entry.cache for entry in entries])
+        states = self.cache.snapshot_state([entry.cache for entry in entries]) if keep_states else []
         try:
             for entry in entries:
                 self.cache.extend(entry.cache, len(entry.tokens))
@@ -629,7 +632,7 @@ class ModelRunner:
 
     decode_steps_sample = True     # decode_steps() also draws from filtered, tempered distributions
 
-    def decode_steps(self, entries: Sequence[StepEntry], steps: int, sampling: Sequence | None = None) -> list[list[int]]:
+    def decode_steps(self, entries: Sequence[StepEntry], steps: int, sampling: Sequence | None = None, keep_states: bool = True) -> list[list[int]]:
         """`steps` decode steps of the same requests, the host out of the loop between them.
 
         Each entry brings the one token its request decodes next.  After every step the device itself
@@ -653,7 +656,7 @@ class ModelRunner:
         if sampling is not None and len(sampling) != len(entries):
             raise GenerationError("decode_steps needs one sampling row per entry")
         before = [entry.cache.length for entry in entries]
-        states = self.cache.snapshot_state([entry.cache for entry in entries])
+        states = self.cache.snapshot_state([entry.cache for entry in entries]) if keep_states else []    # see step()
         chosen: list[list[int]] = []
         current, rows = list(entries), sampling
         try:

@@ -26,7 +26,7 @@ from .loading import load_model, resolve_device, resolve_dtype
 from .step import ModelRunner, StepEntry
 
 PAGE_SIZE = 16
-MAX_LIVE_REQUESTS = 8
+MAX_LIVE_REQUESTS = 4      # state slots (and block table rows): no more requests are live at any time, so slots are used again
 
 
 def build_parser() -> argparse.ArgumentParser:
@@ -37,11 +37,12 @@ def build_parser() -> argparse.ArgumentParser:
     parser.add_argument("--max-tokens", type=int, required=True,
                         help="most tokens that live requests hold at any time; the cache pool is made for this many")
     parser.add_argument("--page-size", type=int, default=PAGE_SIZE)
+    parser.add_argument("--max-requests", type=int, default=MAX_LIVE_REQUESTS, help="most requests that are live at any time")
     return parser
 
 
 def make_runner(model_dir, dtype_name: str, max_tokens: int, page_size: int = PAGE_SIZE, library_gemm: bool = True,
-                use_graph: bool = False):
+                use_graph: bool = False, max_requests: int = MAX_LIVE_REQUESTS):
     device = resolve_device("auto")
     dtype = resolve_dtype(dtype_name)
     # a replay takes the folder as it is: tensors stored in 32-bit beside bfloat16 ones stay 32-bit
@@ -49,7 +50,7 @@ def make_runner(model_dir, dtype_name: str, max_tokens: int, page_size: int = PA
     if max_tokens <= 0:
         raise GenerationError("--max-tokens must be positive")
     num_pages = -(-max_tokens // page_size)
-    cache = CacheManager(model.cache_needs(), page_size=page_size, num_pages=num_pages, max_requests=MAX_LIVE_REQUESTS,
+    cache = CacheManager(model.cache_needs(), page_size=page_size, num_pages=num_pages, max_requests=max_requests,
                          max_seq_len=min(model.spec.max_positions, num_pages * page_size), dtype=dtype, device=device)
     runner = ModelRunner(model, cache, max_step_tokens=num_pages * page_size, dtype=dtype, device=device, library_gemm=library_gemm,
                          use_graph=use_graph)
@@ -83,7 +84,7 @@ def replay(runner: ModelRunner, lines, out_dir: Path, echo=print) -> None:
 
 def main(argv=None) -> int:
     args = build_parser().parse_args(argv)
-    runner = make_runner(args.model, args.dtype, args.max_tokens, args.page_size)
+    runner = make_runner(args.model, args.dtype, args.max_tokens, args.page_size, max_requests=args.max_requests)
     with torch.cuda.device(runner.device):
         replay(runner, sys.stdin, args.out, echo=lambda text: print(text, flush=True))
         torch.cuda.synchronize()

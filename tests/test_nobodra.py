@@ -1,0 +1,139 @@
+"""Nobodra without a GPU: its configuration, the tensors it asks a checkpoint for, what it keeps between steps, and the
+plain implementation's mechanisms against properties that follow from their definitions."""
+
+import json
+import math
+
+import pytest
+import torch
+
+from tests import nobodra_configs as configs
+from tests.plain import nobodra as plain
+
+
+def test_configuration_reads_back_and_names_its_tensors(tmp_path):
+    from llm_runtime_study_amd.config import NobodraConfig, config_from_dict, load_config, spec_for
+    from llm_runtime_study_amd.models import DecoderModel
+    from llm_runtime_study_amd.parts import PagedKVNeed, StateNeed
+
+    for raw in (configs.ROUTED, configs.DENSE, configs.CORES):
+        config = config_from_dict(raw)
+        assert isinstance(config, NobodraConfig) and config.to_json_dict() == raw
+        model = DecoderModel(spec_for(config))
+        names = model.tensors()
+        assert {"embed", "head", "final.norm", "l0.norm1"} <= set(names) and not any(name.endswith(".weight") for name in names)
+        for index, layer in enumerate(raw["layers"]):
+            m, p = layer["mixer"], f"l{index}."
+            if layer["type"] == "attention":
+                assert names[p + "mix.q"].shape == (m["heads"] * m["dim"], raw["width"]) and names[p + "mix.k.norm"].shape == (m["dim"],)
+                assert p + "mix.v" not in names
+            else:
+                assert names[p + "mix.v.conv"].shape == (m["heads"] * m["vdim"], m["conv"]) and names[p + "mix.A_log"].shape == (m["heads"],)
+                assert names[p + "mix.q"].shape == (m["kv_heads"] * m["dim"], raw["width"]) and names[p + "mix.norm"].shape == (m["vdim"],)
+            if layer["mlp"] is None:
+                assert p + "norm2" not in names and not any(name.startswith(p + "mlp.") for name in names)
+            else:
+                last = layer["mlp"]["router"]["experts"] - 1
+                assert names[f"{p}mlp.e{last}.down"].shape == (raw["width"], layer["mlp"]["expert"]["ff"]) and names[p + "mlp.router.b"].shape == (last + 1,)
+        needs = model.cache_needs()
+        for layer, need in zip(raw["layers"], needs):
+            if layer["type"] == "attention":
+                mask = layer["mixer"].get("mask")
+                assert need == PagedKVNeed(layer["mixer"]["kv_heads"], layer["mixer"]["dim"], None if mask is None else mask["size"])
+            else:
+                assert isinstance(need, StateNeed) and need.dtype == torch.float32
+        assert model.graph_safe() and model.plan_safe()
+    folder = configs.write_folder(configs.ROUTED, 3, tmp_path / "m")
+    assert load_config(folder).to_json_dict() == configs.ROUTED
+
+
+def test_what_a_delta_layer_keeps_between_steps():
+    from llm_runtime_study_amd.parts import PartSpec, create
+
+    part = create("mixer", PartSpec("gated_delta_rule", {"hidden_size": 8, "num_heads": 3, "num_kv_heads": 1, "head_dim": 10, "value_dim": 7,
+                                                        "conv_taps": 4, "norm_eps": 1e-6}))
+    # three matrices of 10 (padded to 12) x 7, and the last three inputs of 2 * 10 + 3 * 7 channels
+    assert part.cache_need().shape == (3 * 12 * 7 + 3 * 41,)
+
+
+@pytest.mark.parametrize("broken,message", [
+    (lambda raw: raw["layers"][0].update(type="conv"), "unknown type"),
+    (lambda raw: raw["layers"][1]["mixer"].update(vdim=48), "vdim must equal dim"),
+    (lambda raw: raw["layers"][0]["mixer"].pop("conv"), "conv"),
+    (lambda raw: raw["layers"][1]["mixer"].update(kv_heads=4), "multiple of kv_heads"),
+    (lambda raw: raw["layers"][1]["mlp"]["router"].update(top=9), "exceeds"),
+    (lambda raw: raw["layers"][1]["mixer"]["rot"].update(dims=34), "rot.dims"),
+    (lambda raw: raw.pop("norm"), "norm"),
+    (lambda raw: raw.update(layers=[]), "non-empty"),
+])
+def test_configuration_refuses(broken, message):
+    from llm_runtime_study_amd.config import config_from_dict
+    from llm_runtime_study_amd.errors import ConfigError
+
+    raw = json.loads(json.dumps(configs.ROUTED))
+    broken(raw)
+    with pytest.raises(ConfigError, match=message):
+        config_from_dict(raw)
+
+
+def test_checkpoint_names():
+    from llm_runtime_study_amd.models.nobodra import checkpoint_name
+
+    assert [checkpoint_name(name) for name in ("l3.mix.q_proj.weight", "l3.mix.q_norm.weight", "l0.mix.v_conv.weight", "l0.mix.A_log", "l0.mix.norm.weight",
+                                                "l2.mlp.experts.11.down.weight", "l2.mlp.router.bias", "l2.mlp.router.weight", "final.norm.weight", "embed")] == \
+        ["l3.mix.q", "l3.mix.q.norm", "l0.mix.v.conv", "l0.mix.A_log", "l0.mix.norm", "l2.mlp.e11.down", "l2.mlp.router.b", "l2.mlp.router", "final.norm", "embed"]
+
+
+# ------------------------------------------------------------- the plain mechanisms against their definitions
+def test_plain_delta_rule_recalls_what_it_wrote():
+    """With a full step, no decay and a unit key, reading with the key right after the write gives the value back;
+    the value written under another, orthogonal key is still there."""
+    torch.manual_seed(0)
+    d, e = 6, 5
+    k1, k2 = torch.zeros(d, dtype=torch.float64), torch.zeros(d, dtype=torch.float64)
+    k1[0], k2[3] = 1.0, 1.0
+    v1, v2 = torch.randn(e, dtype=torch.float64), torch.randn(e, dtype=torch.float64)
+    memory = torch.zeros(d, e, dtype=torch.float64)
+    for k, v in ((k1, v1), (k2, v2), (k1, v2)):
+        memory = memory + torch.outer(k, 1.0 * (v - memory.T @ k))
+    torch.testing.assert_close(memory.T @ k1, v2)
+    torch.testing.assert_close(memory.T @ k2, v2)
+
+
+def test_plain_convolution_and_rotation():
+    x = torch.arange(12, dtype=torch.float64).view(6, 2)
+    taps = torch.tensor([[0.0, 0.0, 1.0], [1.0, 0.0, 0.0]], dtype=torch.float64)
+    y = plain.short_convolution(x, taps)
+    torch.testing.assert_close(y[:, 0], x[:, 0])                                        # the last tap is the current token's
+    torch.testing.assert_close(y[:, 1], torch.cat((torch.zeros(2, dtype=torch.float64), x[:4, 1])))      # the first looks two back
+    q = torch.randn(5, 2, 8, dtype=torch.float64)
+    r = plain.rotate_front(q, 100.0, 4)
+    torch.testing.assert_close(r[0], q[0])                                              # position 0 is not turned
+    torch.testing.assert_close(r[..., 4:], q[..., 4:])
+    torch.testing.assert_close(r[..., :4].norm(dim=-1), q[..., :4].norm(dim=-1))
+    angle = 3 * 100.0 ** (-2.0 / 4)
+    torch.testing.assert_close(r[3, 1, 1], q[3, 1, 1] * math.cos(angle) - q[3, 1, 3] * math.sin(angle))
+
+
+def test_plain_window_and_experts():
+    torch.manual_seed(1)
+    n, width, heads, groups, d = 9, 12, 4, 2, 6
+    x = torch.randn(n, width, dtype=torch.float64)
+    w = dict(w_q=torch.randn(heads * d, width, dtype=torch.float64), w_k=torch.randn(groups * d, width, dtype=torch.float64),
+             w_o=torch.randn(width, heads * d, dtype=torch.float64), q_weight=torch.ones(d, dtype=torch.float64), k_weight=torch.ones(d, dtype=torch.float64))
+    full = plain.keys_as_values_attention(x, **w, heads=heads, groups=groups, d=d, eps=1e-6, scale=0.3)
+    wide = plain.keys_as_values_attention(x, **w, heads=heads, groups=groups, d=d, eps=1e-6, scale=0.3, window=n)
+    one = plain.keys_as_values_attention(x, **w, heads=heads, groups=groups, d=d, eps=1e-6, scale=0.3, window=1)
+    torch.testing.assert_close(full, wide)
+    # a window of one sees the token alone: the output is its own key, as projected, through the output matrix
+    alone = (x @ w["w_k"].T).view(n, groups, d).repeat_interleave(heads // groups, 1).reshape(n, heads * d) @ w["w_o"].T
+    torch.testing.assert_close(one, alone)
+    router, bias = torch.randn(4, width, dtype=torch.float64), torch.randn(4, dtype=torch.float64)
+    ups, downs = [torch.randn(5, width, dtype=torch.float64) for _ in range(4)], [torch.randn(width, 5, dtype=torch.float64) for _ in range(4)]
+    every = plain.routed_experts(x, router, bias, ups, downs, 4)
+    share = torch.softmax(x @ router.T + bias, -1)
+    mixture = sum(share[:, e:e + 1] * (torch.relu(x @ ups[e].T).pow(2) @ downs[e].T) for e in range(4))
+    torch.testing.assert_close(every, mixture)
+    best = plain.routed_experts(x, router, bias, ups, downs, 1)
+    chosen = (x @ router.T + bias).argmax(-1)
+    torch.testing.assert_close(best[2], torch.relu(ups[chosen[2]] @ x[2]).pow(2) @ downs[chosen[2]].T)

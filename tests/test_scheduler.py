@@ -22,7 +22,7 @@ class FakeRunner:
                                   max_seq_len=max_seq_len, dtype=torch.float32, device="cpu", allocate_storage=False)
         self.script, self.produced, self.calls, self.fail_at = script, {}, [], None
 
-    def step(self, entries):
+    def step(self, entries, keep_states=True):
         if self.fail_at is not None and len(self.calls) == self.fail_at:
             raise RuntimeError("injected failure")
         self.calls.append([(e.cache.request_id, list(e.tokens), list(e.want)) for e in entries])
@@ -220,7 +220,7 @@ class SeveralStepsRunner(FakeRunner):
     def can_decode_steps(self, entries):
         return all(len(e.tokens) == 1 for e in entries)
 
-    def decode_steps(self, entries, steps, sampling=None):
+    def decode_steps(self, entries, steps, sampling=None, keep_states=True):
         self.launches.append((steps, [e.cache.request_id for e in entries]))
         self.sampling_seen.append(None if sampling is None else [(row.config.temperature, row.seed, row.counter) for row in sampling])
         chosen = []
@@ -298,7 +298,7 @@ class QueuedLaunchRunner(SeveralStepsRunner):
         self.begun, self.ended, self.dropped, self.serial, self.open = [], [], [], 0, 0
         self.decode_steps_sample = True
 
-    def step(self, entries):
+    def step(self, entries, keep_states=True):
         assert self.open == 0, "a step ran while a launch was in flight"
         self.serial += 1
         return super().step(entries)
