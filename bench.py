@@ -1,6 +1,7 @@
 """Decode and prefill throughput of the Qwen3-8B shape with random weights on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 2048] [--layers L] [--shape 8b|14b|32b]
+    python bench.py --design nobodra [--shape 8b] [--layers 8] ...     # the Nobodra design at the shape's layer sizes, beside the shape itself
 
 A step is one decode step of the whole engine (scheduler, step function, sampling) at the
 given batch; `value` is decoded tokens per second.  The same line carries the prefill rate
@@ -25,7 +26,7 @@ if str(ROOT) not in sys.path:
 HBM_PEAK = 8.0e12
 FLOP_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
 
-from llm_runtime_study_amd.benchmarks.shapes import QWEN3_8B, SHAPES  # noqa: E402  (layer sizes of the 8B, 14B and 32B models)
+from llm_runtime_study_amd.benchmarks.shapes import QWEN3_8B, SHAPES, nobodra_like  # noqa: E402  (layer sizes of the 8B, 14B and 32B models)
 
 FULL_LAYERS = QWEN3_8B["num_hidden_layers"]
 BENCHMARK_CONTEXT = 4096      # tokens a request's cache can hold at the least: the benchmark context of the 8B configuration
@@ -45,6 +46,8 @@ def parse_args():
     parser.add_argument("--num-pages", type=int, default=None, help="pages of the cache pool (default: max-seq-len tokens for every request of the largest batch)")
     parser.add_argument("--shape", choices=tuple(SHAPES), default="8b", help="layer sizes: Qwen3-8B (default), 14B or 32B")
     parser.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (reported in config)")
+    parser.add_argument("--design", choices=("qwen3", "nobodra"), default="qwen3",
+                        help="nobodra: measure that design at the shape's layer sizes (8 layers unless --layers says otherwise) and, beside it, the shape itself with as many layers")
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points")
     parser.add_argument("--temperature", type=float, default=0.0, help="draw the tokens at this temperature instead of taking the largest logit (reported in config)")
@@ -180,11 +183,99 @@ def prefill_entry(engine, tokens: int, dtype_name: str, seed: int) -> dict:
             "frac": round(prefill_flops(engine.model, tokens) / seconds / FLOP_PEAK[dtype_name], 4)}
 
 
+def step_bytes(engine, batch: int, mean_context: float) -> float:
+    """Bytes a decode step of `batch` requests must read (and, for states, write back): the weights in use, the cached
+    keys and values inside every layer's window, every request's state rows.  A layer of routed experts reads the experts
+    that the batch's tokens choose between them: experts * (1 - (1 - top / experts) ** batch) of them on average."""
+    import math
+
+    from llm_runtime_study_amd.parts import PagedKVNeed, StateNeed
+
+    model, total = engine.model, 0.0
+    for entry, need in zip(model.spec.schedule, model.cache_needs()):
+        layer = model.layers[entry.layer]
+        total += layer.weight_bytes()
+        ff = getattr(layer, "feed_forward", None)
+        if ff is not None and hasattr(ff, "num_experts"):
+            hit = ff.num_experts * (1.0 - (1.0 - ff.top / ff.num_experts) ** batch)
+            total += (hit - ff.top) * 2 * ff.hidden_size * ff.intermediate_size * ff.up.element_size()
+        if isinstance(need, PagedKVNeed):
+            held = mean_context if need.window is None else min(mean_context, need.window)
+            total += 2 * batch * held * need.num_kv_heads * need.head_dim * (2 if engine.dtype == torch_bfloat16() else 4)
+        elif isinstance(need, StateNeed):
+            total += 2 * batch * math.prod(need.shape) * 4
+    return total + model.head.numel() * model.head.element_size()
+
+
+def torch_bfloat16():
+    import torch
+
+    return torch.bfloat16
+
+
+def measure_design(args, config, dtype_name: str, max_seq_len: int, max_batch: int) -> dict:
+    """Prefill and decode figures of one engine made from `config` with random weights."""
+    from llm_runtime_study_amd import Engine
+    from llm_runtime_study_amd.kernels.ops import KernelChoice
+
+    engine = Engine.from_config(config, seed=0, dtype=args.dtype, max_seq_len=max_seq_len, max_batch_size=max_batch,
+                                max_num_batched_tokens=max(2048, args.prefill_tokens), use_cuda_graph=not args.no_graph, num_pages=args.num_pages,
+                                kernels=KernelChoice(library=not args.own_gemm, mid=not args.library_mid_gemm),
+                                decode_steps_per_launch=args.decode_steps_per_launch, launch_ahead=not args.no_launch_ahead,
+                                reserve_memory=not args.no_reserve)
+    out = {"prefill": prefill_entry(engine, args.prefill_tokens, dtype_name, seed=1), f"prefill_{PORTION_TOKENS}": prefill_entry(engine, PORTION_TOKENS, dtype_name, seed=5)}
+    for batch in sorted({1, args.batch, max_batch}):
+        steps = args.steps if batch == args.batch else min(args.steps, 64)
+        times, mean_context = measure_decode(engine, batch, args.context, steps, min(args.warmup, 4), seed=2 + batch)
+        step_s = sum(times) / len(times)
+        moved = step_bytes(engine, batch, mean_context)
+        out[f"decode_b{batch}"] = {"tok_s": round(batch / step_s, 2), "ms_per_step": round(step_s * 1e3, 4), "GB_per_step": round(moved / 1e9, 3),
+                                   "hbm_frac": round(moved / step_s / HBM_PEAK, 4)}
+    engine.runner.drop_graphs()
+    return out
+
+
+def design_main(args) -> int:
+    """--design nobodra: the design at the shape's layer sizes, and the shape itself with as many layers, one after the other."""
+    import gc
+
+    import torch
+
+    from llm_runtime_study_amd.config import config_from_dict
+
+    layers = args.layers or 8
+    dtype_name = "bf16" if args.dtype == "bfloat16" else "fp32"
+    max_batch = args.batch if args.no_points else max(args.batch, 64)
+    max_seq_len = args.max_seq_len or max(BENCHMARK_CONTEXT, args.context + args.steps + warmup_room(args.warmup, max(args.decode_steps_per_launch, 1))
+                                          + decode_lead(max_batch, args.context, max(2048, args.prefill_tokens)) + max_batch + 64, args.prefill_tokens + 1)
+    raw = nobodra_like(SHAPES[args.shape], layers)
+    mine = measure_design(args, config_from_dict(raw), dtype_name, max_seq_len, max_batch)
+    gc.collect()
+    torch.cuda.empty_cache()
+    beside = measure_design(args, config_from_dict(dict(SHAPES[args.shape], num_hidden_layers=layers)), dtype_name, max_seq_len, max_batch)
+    main_point = mine[f"decode_b{args.batch}"]
+    line = {
+        "metric": f"decode tok/s at batch {args.batch} (Nobodra at Qwen3-{args.shape.upper()} layer sizes, {layers} layers)",
+        "value": main_point["tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": main_point["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype_name,
+        "data": "synthetic (seeded uniform random token ids, random weights N(0, 0.02))",
+        "config": {"model": f"Nobodra at Qwen3-{args.shape.upper()} layer sizes", "layers": layers, "width": raw["width"], "layer_kinds": [layer["type"] for layer in raw["layers"]],
+                   "mixer": raw["layers"][-1]["mixer"] if layers >= 4 else raw["layers"][0]["mixer"], "delta_mixer": raw["layers"][0]["mixer"], "mlp": raw["layers"][0]["mlp"],
+                   "global_batch": args.batch, "seq_len": args.context, "max_seq_len": max_seq_len, "prefill_tokens": args.prefill_tokens, "parallelism": "single GPU"},
+        "nobodra": mine,
+        "beside": {"model": f"Qwen3-{args.shape.upper()} shape, {layers} layers", **beside},
+    }
+    print(json.dumps(line))
+    return 0
+
+
 def main() -> int:
     args = parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU only: --gpus {args.gpus} is not supported by this single-GPU engine")
         return 2
+    if args.design != "qwen3":
+        return design_main(args)
     import torch
 
     from llm_runtime_study_amd import Engine

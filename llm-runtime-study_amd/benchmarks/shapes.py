@@ -16,3 +16,18 @@ SHAPES = {
     "14b": dict(QWEN3_8B, hidden_size=5120, intermediate_size=17408, num_hidden_layers=40, num_attention_heads=40),
     "32b": dict(QWEN3_8B, hidden_size=5120, intermediate_size=25600, num_hidden_layers=64, num_attention_heads=64),
 }
+
+
+def nobodra_like(shape: dict, layers: int, experts: int = 32, top: int = 8, window: int = 4096) -> dict:
+    """A Nobodra configuration with the layer sizes of a dense shape above, for measurements beside it: the same width,
+    vocabulary and heads; three gated-delta-rule layers to every sliding-window attention layer; the dense feed-forward's
+    three matrices of `intermediate_size` as `top` of `experts` experts of two matrices each with as many weights in use
+    per token (to a multiple of 128); half of every attention head rotated."""
+    width, heads, kv_heads, dim = shape["hidden_size"], shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"]
+    ff = max(128, round(3 * shape["intermediate_size"] / (2 * top) / 128) * 128)
+    mlp = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
+    attention = {"type": "attention", "mlp": mlp, "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                                                            "mask": {"size": window}, "rot": {"base": 1000000.0, "dims": dim // 2}}}
+    delta = {"type": "delta", "mlp": mlp, "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "conv": 4}}
+    return {"architecture": "Nobodra", "vocab": shape["vocab_size"], "width": width, "norm": {"eps": 1e-6},
+            "layers": [attention if index % 4 == 3 else delta for index in range(layers)]}

@@ -111,9 +111,9 @@ enum { ACT_NONE = 0, ACT_RELU_SQUARED = 1 };
 template <typename T, typename TO>
 __global__ __launch_bounds__(256) void moe_experts_kernel(TO* __restrict__ out, int ldc, const T* __restrict__ a, int lda,
                                                           const T* __restrict__ w, int n, int k, const int* __restrict__ sorted,
-                                                          const int* __restrict__ tile_expert, int top, int gather, int act) {
+                                                          const int* __restrict__ tile_expert, int top, int gather, int act, int sub) {
   constexpr int TM = 32, TN = 64, TK = 16;
-  const int expert = tile_expert[blockIdx.x];
+  const int expert = tile_expert[blockIdx.x / sub];       // sub: runs of 32 rows in a tile of the sorted list
   if (expert < 0) return;
   __shared__ float a_s[TK][TM + 1];
   __shared__ float b_s[TK][TN + 1];
@@ -248,6 +248,88 @@ __global__ __launch_bounds__(256) void moe_experts_bf16_kernel(TO* __restrict__ 
   }
 }
 
+// The same for steps that bring an expert a hundred rows and more: 128 rows x 128 columns per workgroup, a wave
+// 64 x 64 as four by four products, so that a slice of K is fetched once for four times the work.
+constexpr int WM = 128;
+
+template <typename TO>
+__global__ __launch_bounds__(256) void moe_experts_bf16_wide_kernel(TO* __restrict__ out, int ldc, const bf16* __restrict__ a, int lda,
+                                                                    const bf16* __restrict__ w, int n, int k, const int* __restrict__ sorted,
+                                                                    const int* __restrict__ tile_expert, int top, int gather, int act) {
+  const int expert = tile_expert[blockIdx.x];
+  if (expert < 0) return;
+  __shared__ __attribute__((aligned(16))) bf16 a_s[WM][GK + GPAD];
+  __shared__ __attribute__((aligned(16))) bf16 b_s[GN][GK + GPAD];
+  __shared__ int row_of[WM];
+  const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+  const int row0 = blockIdx.x * WM, col0 = blockIdx.y * GN;
+  if (tid < WM) {
+    const int pair = sorted[row0 + tid];
+    row_of[tid] = pair < 0 ? -1 : (gather ? pair / top : row0 + tid);
+  }
+  __syncthreads();
+  const bf16* we = w + (int64_t)expert * n * k;
+  const int l_row = tid / 8, l_col = (tid % 8) * 8;          // a thread brings 16 bytes of rows l_row, + 32, + 64, + 96
+  const bf16* a_ptr[4];
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    const int src = row_of[p * 32 + l_row];
+    a_ptr[p] = src >= 0 ? a + (int64_t)src * lda + l_col : nullptr;
+  }
+  bf16x8 a_reg[4], b_reg[4];
+  const bf16x8 zero = {};
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      a_reg[p] = a_ptr[p] ? *(const bf16x8*)(a_ptr[p] + k0) : zero;
+      const int r = p * 32 + l_row;
+      b_reg[p] = col0 + r < n ? *(const bf16x8*)(we + (int64_t)(col0 + r) * k + k0 + l_col) : zero;
+    }
+  };
+  floatx4 acc[4][4] = {};
+  fetch(0);
+  const int wm = wave / 2, wn = wave % 2, frag_row = lane % 16, frag_k = (lane / 16) * 8;
+  for (int k0 = 0; k0 < k; k0 += GK) {
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      *(bf16x8*)&a_s[p * 32 + l_row][l_col] = a_reg[p];
+      *(bf16x8*)&b_s[p * 32 + l_row][l_col] = b_reg[p];
+    }
+    __syncthreads();
+    if (k0 + GK < k) fetch(k0 + GK);
+#pragma unroll
+    for (int kk = 0; kk < GK; kk += 32) {
+      bf16x8 af[4], bfr[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) af[i] = *(const bf16x8*)&a_s[wm * 64 + i * 16 + frag_row][kk + frag_k];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) bfr[i] = *(const bf16x8*)&b_s[wn * 64 + i * 16 + frag_row][kk + frag_k];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj)
+          acc[i][jj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bfr[jj], af[i], acc[i][jj], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = wm * 64 + i * 16 + lane % 16;
+    if (row_of[m] < 0) continue;
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+      const int c = col0 + wn * 64 + jj * 16 + (lane / 16) * 4;
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        if (c + x >= n) continue;
+        float v = acc[i][jj][x];
+        if (act == ACT_RELU_SQUARED) v = v > 0.f ? v * v : 0.f;
+        out[(int64_t)(row0 + m) * ldc + c + x] = from_float<TO>(v);
+      }
+    }
+  }
+}
+
 template <typename TW>
 __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ residual, const float* __restrict__ rows, int hidden,
                                                           const int* __restrict__ place, const float* __restrict__ weights, int top,
@@ -274,12 +356,14 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ re
 
 }  // namespace
 
-LRS_API int lrs_moe_tile_rows() { return 32; }
+// Rows of a tile of the grouped products: 32, or 128 once the step brings every expert 128 rows and more on average
+// (follows from the step's shape alone, so that recorded and captured steps keep it).
+LRS_API int lrs_moe_tile_rows(int pairs, int experts) { return (int64_t)pairs >= (int64_t)WM * experts ? WM : GM; }
 
 // The most tiles that `pairs` (token, choice) pairs of `experts` experts can fill: every expert in use ends in at
 // most one tile that is not full.
 LRS_API int lrs_moe_max_tiles(int pairs, int experts) {
-  const int padded = pairs / lrs_moe_tile_rows() + experts;
+  const int padded = pairs / lrs_moe_tile_rows(pairs, experts) + experts;
   return pairs < padded ? pairs : padded;
 }
 
@@ -294,8 +378,8 @@ LRS_API int lrs_moe_route(const float* logits, int ld, const float* bias, int* i
 
 LRS_API int lrs_moe_align(const int* ids, int pairs, int experts, int* sorted, int capacity, int* place, int* tile_expert,
                           int max_tiles, void* stream) {
-  const int tile = lrs_moe_tile_rows();
   LRS_REQUIRE(pairs > 0 && experts > 0, "moe_align: bad sizes pairs=%d experts=%d", pairs, experts);
+  const int tile = lrs_moe_tile_rows(pairs, experts);
   LRS_REQUIRE(max_tiles >= lrs_moe_max_tiles(pairs, experts), "moe_align: %d tiles may not hold %d pairs of %d experts", max_tiles, pairs, experts);
   LRS_REQUIRE(capacity >= max_tiles * tile, "moe_align: the sorted list holds %d rows, %d tiles need %d", capacity, max_tiles, max_tiles * tile);
   const size_t lds = (size_t)(3 * experts + 1) * sizeof(int);
@@ -307,12 +391,23 @@ LRS_API int lrs_moe_align(const int* ids, int pairs, int experts, int* sorted, i
 // out [max_tiles * tile, n] = rows of `a` (row pair / top of the sorted list if `gather`, else the sorted row
 // itself) times the tile's expert matrix w[expert] [n, k], transposed; act 1: the square of relu.
 LRS_API int lrs_moe_experts(void* out, int out_dtype, int ldc, const void* a, const void* w, int dtype, int lda, int n, int k,
-                            const int* sorted, const int* tile_expert, int max_tiles, int top, int gather, int act, void* stream) {
+                            const int* sorted, const int* tile_expert, int max_tiles, int tile, int top, int gather, int act, void* stream) {
+  LRS_REQUIRE(tile == GM || tile == WM, "moe_experts: tiles have %d or %d rows, got %d", GM, WM, tile);
   LRS_REQUIRE(max_tiles > 0 && n > 0 && k > 0 && top > 0, "moe_experts: bad sizes tiles=%d n=%d k=%d top=%d", max_tiles, n, k, top);
   LRS_REQUIRE(lda >= k && ldc >= n, "moe_experts: strides lda=%d ldc=%d too small for k=%d n=%d", lda, ldc, k, n);
   LRS_REQUIRE(act == ACT_NONE || act == ACT_RELU_SQUARED, "moe_experts: unknown activation %d", act);
   hipStream_t s = (hipStream_t)stream;
   const bool cores = dtype == LRS_BF16 && k % GK == 0 && lda % 8 == 0 && ((uintptr_t)a % 16) == 0 && ((uintptr_t)w % 16) == 0;
+  if (cores && tile == WM) {
+    dim3 grid(max_tiles, (n + GN - 1) / GN);
+    if (out_dtype == LRS_BF16)
+      moe_experts_bf16_wide_kernel<bf16><<<grid, 256, 0, s>>>((bf16*)out, ldc, (const bf16*)a, lda, (const bf16*)w, n, k, sorted, tile_expert, top, gather, act);
+    else if (out_dtype == LRS_F32)
+      moe_experts_bf16_wide_kernel<float><<<grid, 256, 0, s>>>((float*)out, ldc, (const bf16*)a, lda, (const bf16*)w, n, k, sorted, tile_expert, top, gather, act);
+    else
+      return lrs_fail("moe_experts: unknown output dtype %d", out_dtype);
+    return lrs_check_launch("moe_experts");
+  }
   if (cores) {
     dim3 grid(max_tiles, (n + GN - 1) / GN);
     if (out_dtype == LRS_BF16)
@@ -323,8 +418,8 @@ LRS_API int lrs_moe_experts(void* out, int out_dtype, int ldc, const void* a, co
       return lrs_fail("moe_experts: unknown output dtype %d", out_dtype);
     return lrs_check_launch("moe_experts");
   }
-  dim3 grid(max_tiles, (n + 63) / 64);
-#define RUN(T, TO) moe_experts_kernel<T, TO><<<grid, 256, 0, s>>>((TO*)out, ldc, (const T*)a, lda, (const T*)w, n, k, sorted, tile_expert, top, gather, act)
+  dim3 grid(max_tiles * (tile / GM), (n + 63) / 64);       // the any-shape form walks a tile of 128 rows as four of 32
+#define RUN(T, TO) moe_experts_kernel<T, TO><<<grid, 256, 0, s>>>((TO*)out, ldc, (const T*)a, lda, (const T*)w, n, k, sorted, tile_expert, top, gather, act, tile / GM)
   if (dtype == LRS_F32 && out_dtype == LRS_F32) RUN(float, float);
   else if (dtype == LRS_BF16 && out_dtype == LRS_BF16) RUN(bf16, bf16);
   else if (dtype == LRS_BF16 && out_dtype == LRS_F32) RUN(bf16, float);

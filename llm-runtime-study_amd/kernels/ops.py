@@ -148,12 +148,12 @@ _SIGNATURES = {
     "lrs_norm_add": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_void_p]),
     "lrs_delta_state_rows": (c_int, [c_int]),
     "lrs_delta_rule": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
-                               c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p]),
-    "lrs_moe_tile_rows": (c_int, []),
+                               c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "lrs_moe_tile_rows": (c_int, [c_int, c_int]),
     "lrs_moe_max_tiles": (c_int, [c_int, c_int]),
     "lrs_moe_route": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "lrs_moe_align": (c_int, [c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p]),
-    "lrs_moe_experts": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int,
+    "lrs_moe_experts": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
                                 c_int, c_int, c_void_p]),
     "lrs_moe_combine": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_float, c_void_p]),
 }
@@ -1128,14 +1128,15 @@ def filter_logits(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.
 # ------------------------------------------------------------------- gated delta rule
 def delta_state_floats(heads: int, kv_heads: int, dim: int, vdim: int, taps: int) -> int:
     """Floats of one request's state row of a gated-delta-rule mixer: the matrix of every head in the order the scan
-    holds it (dim padded to a multiple of four), then the convolution's last taps - 1 inputs of every channel."""
+    holds it (dim padded to 16 lanes of 4, 8 or 16 rows), then the convolution's last taps - 1 inputs of every channel."""
     rows = library().lrs_delta_state_rows(dim)
-    return heads * rows * 4 * vdim + (taps - 1) * (2 * kv_heads * dim + heads * vdim)
+    return heads * rows * 16 * vdim + (taps - 1) * (2 * kv_heads * dim + heads * vdim)
 
 
 def delta_rule(out: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, token_request: torch.Tensor, cu_seqlens: torch.Tensor,
                slot_ids: torch.Tensor, requests: int, conv_weight: torch.Tensor, kv_heads: int, heads: int, dim: int, vdim: int,
-               a_log: torch.Tensor, dt_bias: torch.Tensor, norm_weight: torch.Tensor, eps: float, qkv: torch.Tensor, gates: torch.Tensor) -> None:
+               a_log: torch.Tensor, dt_bias: torch.Tensor, norm_weight: torch.Tensor, eps: float, qkv: torch.Tensor, gates: torch.Tensor,
+               raw: torch.Tensor) -> None:
     """One step of the gated delta rule for a ragged batch.  proj [T, >= C] holds each token's projections, columns
     q (kv_heads*dim) | k (kv_heads*dim) | v (heads*vdim) | output gate (heads*vdim) | step size (heads) | decay input
     (heads); state [slots, floats] float32 is read and written at the rows slot_ids names; out [T, heads*vdim]."""
@@ -1154,21 +1155,23 @@ def delta_rule(out: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, token
         _need(t.dtype == torch.int32 and t.numel() >= count and t.is_contiguous(), f"delta_rule: {name} must be int32 [{count}]")
     _need(qkv.dtype == torch.float32 and qkv.is_contiguous() and qkv.numel() >= tokens * channels, "delta_rule: qkv scratch too small")
     _need(gates.dtype == torch.float32 and gates.is_contiguous() and gates.numel() >= tokens * 2 * heads, "delta_rule: gates scratch too small")
+    _need(raw.dtype == torch.float32 and raw.is_contiguous() and raw.numel() >= tokens * heads * vdim, "delta_rule: read-out scratch too small")
     _launch("lrs_delta_rule", _dev(out, "out"), dtype_code(out.dtype), _dev(proj, "proj"), dtype_code(proj.dtype), _rows(proj, "proj"), tokens,
             requests, _dev(token_request, "token_request"), _dev(cu_seqlens, "cu_seqlens"), _dev(slot_ids, "slot_ids"), _dev(state, "state"),
             state.stride(0), _dev(conv_weight, "conv_weight"), taps, kv_heads, heads, dim, vdim, _dev(a_log, "a_log"), _dev(dt_bias, "dt_bias"),
-            _dev(norm_weight, "norm_weight"), eps, _dev(qkv, "qkv"), _dev(gates, "gates"), _stream())
+            _dev(norm_weight, "norm_weight"), eps, _dev(qkv, "qkv"), _dev(gates, "gates"), _dev(raw, "raw"), _stream())
 
 
 # ------------------------------------------------------------------- routed experts
-@functools.lru_cache(maxsize=1)
-def moe_tile_rows() -> int:
-    return library().lrs_moe_tile_rows()
+def moe_tile_rows(pairs: int, experts: int) -> int:
+    """Rows of a tile of the grouped products for a step of `pairs` (token, choice) pairs: 32, or 128 once every expert
+    gets 128 rows and more on average."""
+    return 128 if pairs >= 128 * experts else 32
 
 
 def moe_max_tiles(pairs: int, experts: int) -> int:
     """The most row tiles that `pairs` (token, choice) pairs of `experts` experts fill once sorted by expert."""
-    return min(pairs, pairs // moe_tile_rows() + experts)
+    return min(pairs, pairs // moe_tile_rows(pairs, experts) + experts)
 
 
 def moe_route(logits: torch.Tensor, bias: torch.Tensor | None, ids: torch.Tensor, weights: torch.Tensor) -> None:
@@ -1187,26 +1190,29 @@ def moe_align(ids: torch.Tensor, experts: int, sorted_pairs: torch.Tensor, place
     """Sorts the (token, choice) pairs of ids [T, top] by expert: sorted_pairs [tiles * tile rows] (pair index, -1 in the
     rows that pad an expert's run), place [T * top] (the row of each pair), tile_expert [tiles] (-1: tile not in use)."""
     pairs, tiles = ids.numel(), tile_expert.numel()
+    tile = moe_tile_rows(pairs, experts)
     for name, t in (("ids", ids), ("sorted_pairs", sorted_pairs), ("place", place), ("tile_expert", tile_expert)):
         _need(t.dtype == torch.int32 and t.is_contiguous(), f"moe_align: {name} must be contiguous int32")
-    _need(tiles >= moe_max_tiles(pairs, experts) and sorted_pairs.numel() >= tiles * moe_tile_rows() and place.numel() >= pairs,
+    _need(tiles >= moe_max_tiles(pairs, experts) and sorted_pairs.numel() >= tiles * tile and place.numel() >= pairs,
           "moe_align: the lists are too short for the step")
     _launch("lrs_moe_align", _dev(ids, "ids"), pairs, experts, _dev(sorted_pairs, "sorted_pairs"), sorted_pairs.numel(), _dev(place, "place"),
             _dev(tile_expert, "tile_expert"), tiles, _stream())
 
 
-def moe_experts(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, sorted_pairs: torch.Tensor, tile_expert: torch.Tensor, top: int,
+def moe_experts(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, sorted_pairs: torch.Tensor, tile_expert: torch.Tensor, tile: int, top: int,
                 gather: bool, relu_squared: bool) -> None:
     """out [tiles * tile rows, N] = rows of `a` times w[expert of the tile] [N, K], transposed, for every tile in use.
+    tile: rows of a tile, as moe_tile_rows() gave them for the step that was sorted.
     gather: the row of a sorted pair is a[pair // top] (tokens); else `a` is in sorted order itself."""
     experts, n, k = w.shape
     tiles = tile_expert.numel()
+    _need(tile in (32, 128), "moe_experts: tiles have 32 or 128 rows")
     _need(w.is_contiguous() and a.dtype == w.dtype and a.shape[1] == k, "moe_experts: a [*, K] and w [E, N, K] must agree")
-    _need(out.shape == (tiles * moe_tile_rows(), n) and out.dtype in (w.dtype, torch.float32), "moe_experts: out must be [tiles * tile rows, N]")
-    _need(gather or a.shape[0] >= tiles * moe_tile_rows(), "moe_experts: sorted rows missing")
-    _need(sorted_pairs.numel() >= tiles * moe_tile_rows(), "moe_experts: sorted list too short")
+    _need(out.shape == (tiles * tile, n) and out.dtype in (w.dtype, torch.float32), "moe_experts: out must be [tiles * tile rows, N]")
+    _need(gather or a.shape[0] >= tiles * tile, "moe_experts: sorted rows missing")
+    _need(sorted_pairs.numel() >= tiles * tile, "moe_experts: sorted list too short")
     _launch("lrs_moe_experts", _dev(out, "out"), dtype_code(out.dtype), _rows(out, "out"), _dev(a, "a"), _dev(w, "w"), dtype_code(w.dtype),
-            _rows(a, "a"), n, k, _dev(sorted_pairs, "sorted_pairs", torch.int32), _dev(tile_expert, "tile_expert", torch.int32), tiles, top,
+            _rows(a, "a"), n, k, _dev(sorted_pairs, "sorted_pairs", torch.int32), _dev(tile_expert, "tile_expert", torch.int32), tiles, tile, top,
             int(gather), int(relu_squared), _stream())
 
 

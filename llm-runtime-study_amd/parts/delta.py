@@ -24,7 +24,12 @@ from ..kernels import ops
 from .base import Part, StateNeed, TensorSpec, register
 from .linear import linear, materialize, rows_of
 
-STATE_LANES = 4      # lanes that share a column of a head's matrix in the scan kernel; head_dim is padded to a multiple of it
+STATE_LANES = 16     # lanes that share a column of a head's matrix in the scan kernel
+
+
+def state_rows(head_dim: int) -> int:
+    """Rows of a head's matrix that one of those lanes holds: head_dim is padded to 16 times 4, 8 or 16."""
+    return 4 if head_dim <= 64 else 8 if head_dim <= 128 else 16
 
 
 class GatedDeltaRule(Part):
@@ -39,8 +44,8 @@ class GatedDeltaRule(Part):
                 raise ValueError(f"{name} must be positive, got {value}")
         if num_heads % num_kv_heads != 0:
             raise ValueError(f"num_heads must be divisible by num_kv_heads, got {num_heads} and {num_kv_heads}")
-        if head_dim > 256 or value_dim > 256:
-            raise ValueError(f"the scan kernel takes head_dim and value_dim up to 256, got {head_dim} and {value_dim}")
+        if head_dim > 256:
+            raise ValueError(f"the scan kernel takes head_dim up to 256, got {head_dim}")
         if norm_eps <= 0:
             raise ValueError(f"norm_eps must be positive, got {norm_eps}")
         self.hidden_size, self.num_heads, self.num_kv_heads = hidden_size, num_heads, num_kv_heads
@@ -82,8 +87,7 @@ class GatedDeltaRule(Part):
         return super().flops(tokens, pairs) + 6.0 * tokens * self.num_heads * self.head_dim * self.value_dim
 
     def state_floats(self) -> int:
-        rows = -(-self.head_dim // STATE_LANES)
-        return self.num_heads * rows * STATE_LANES * self.value_dim + (self.conv_taps - 1) * self.channels
+        return self.num_heads * state_rows(self.head_dim) * STATE_LANES * self.value_dim + (self.conv_taps - 1) * self.channels
 
     def cache_need(self):
         return StateNeed((self.state_floats(),), torch.float32)
@@ -98,8 +102,9 @@ class GatedDeltaRule(Part):
         out = ctx.scratch("delta_out", (t, self.num_heads * self.value_dim), ctx.dtype)
         qkv = ctx.scratch("delta_qkv", (t, self.channels), torch.float32)
         gates = ctx.scratch("delta_gates", (t, 2 * self.num_heads), torch.float32)
+        raw = ctx.scratch("delta_read_out", (t, self.num_heads * self.value_dim), torch.float32)
         ops.delta_rule(out, proj, cache.state, ctx.token_request, ctx.cu_seqlens_q, ctx.slot_ids, ctx.R, self.conv, self.num_kv_heads,
-                       self.num_heads, self.head_dim, self.value_dim, self.a_log, self.dt_bias, self.norm, self.norm_eps, qkv, gates)
+                       self.num_heads, self.head_dim, self.value_dim, self.a_log, self.dt_bias, self.norm, self.norm_eps, qkv, gates, raw)
         linear(ctx, residual, out, self.w_o, accumulate=accumulate)
         return None
 

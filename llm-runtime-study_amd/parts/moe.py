@@ -78,16 +78,16 @@ class RoutedExperts(Part):
         ids = ctx.scratch("moe_ids", (t, top), torch.int32)
         weights = ctx.scratch("moe_weights", (t, top), torch.float32)
         ops.moe_route(logits[:, :experts], self.bias, ids, weights)
-        tiles = ops.moe_max_tiles(t * top, experts)
-        rows = tiles * ops.moe_tile_rows()
+        tile, tiles = ops.moe_tile_rows(t * top, experts), ops.moe_max_tiles(t * top, experts)
+        rows = tiles * tile
         sorted_pairs = ctx.scratch("moe_sorted", (rows,), torch.int32)
         place = ctx.scratch("moe_place", (t * top,), torch.int32)
         tile_expert = ctx.scratch("moe_tile_expert", (tiles,), torch.int32)
         ops.moe_align(ids, experts, sorted_pairs, place, tile_expert)
         hidden = ctx.scratch("moe_hidden", (rows, self.intermediate_size), ctx.dtype)
-        ops.moe_experts(hidden, x, self.up, sorted_pairs, tile_expert, top, gather=True, relu_squared=True)
+        ops.moe_experts(hidden, x, self.up, sorted_pairs, tile_expert, tile, top, gather=True, relu_squared=True)
         outputs = ctx.scratch("moe_outputs", (rows, self.hidden_size), torch.float32)
-        ops.moe_experts(outputs, hidden, self.down, sorted_pairs, tile_expert, top, gather=False, relu_squared=False)
+        ops.moe_experts(outputs, hidden, self.down, sorted_pairs, tile_expert, tile, top, gather=False, relu_squared=False)
         if output_norm is None:
             ops.moe_combine(residual, outputs, place, weights, None)
         else:

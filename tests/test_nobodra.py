@@ -52,8 +52,8 @@ def test_what_a_delta_layer_keeps_between_steps():
 
     part = create("mixer", PartSpec("gated_delta_rule", {"hidden_size": 8, "num_heads": 3, "num_kv_heads": 1, "head_dim": 10, "value_dim": 7,
                                                         "conv_taps": 4, "norm_eps": 1e-6}))
-    # three matrices of 10 (padded to 12) x 7, and the last three inputs of 2 * 10 + 3 * 7 channels
-    assert part.cache_need().shape == (3 * 12 * 7 + 3 * 41,)
+    # three matrices of 10 (padded to 16 lanes of 4 rows) x 7, and the last three inputs of 2 * 10 + 3 * 7 channels
+    assert part.cache_need().shape == (3 * 64 * 7 + 3 * 41,)
 
 
 @pytest.mark.parametrize("broken,message", [

@@ -63,7 +63,7 @@ def test_gated_delta_rule_part(dtype, heads, groups, d, e, taps):
     w["A_log"] = (w["A_log"] - 2.0).to(torch.bfloat16).double()      # decays near one: what a token wrote is still there dozens of tokens on
     w["norm.weight"] = (w["norm.weight"] + 1.0).to(torch.bfloat16).double()
     part.bind({name: t.to(torch.bfloat16).cuda() for name, t in w.items()}, dtype)
-    assert part.state_floats() == heads * ops.library().lrs_delta_state_rows(d) * 4 * e + (taps - 1) * (2 * groups * d + heads * e)
+    assert part.state_floats() == heads * ops.library().lrs_delta_state_rows(d) * 16 * e + (taps - 1) * (2 * groups * d + heads * e)
     named = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "q.conv": "q_conv.weight", "k.conv": "k_conv.weight",
              "v.conv": "v_conv.weight", "b": "b_proj.weight", "a": "a_proj.weight", "A_log": "A_log", "dt_bias": "dt_bias", "g": "g_proj.weight",
              "norm": "norm.weight", "o": "o_proj.weight"}
@@ -104,7 +104,8 @@ def moe_weights(width, ff, count, seed):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("width,ff,count,top,tokens", [(64, 48, 6, 2, 50), (128, 64, 70, 3, 200), (128, 128, 8, 8, 33), (40, 24, 5, 1, 7), (192, 64, 16, 4, 1)])
+@pytest.mark.parametrize("width,ff,count,top,tokens", [(64, 48, 6, 2, 50), (128, 64, 70, 3, 200), (128, 128, 8, 8, 33), (40, 24, 5, 1, 7), (192, 64, 16, 4, 1),
+                                                       (128, 192, 3, 2, 300), (72, 40, 2, 2, 260)])
 def test_grouped_expert_products_with_given_choices(dtype, width, ff, count, top, tokens):
     """The sort by expert, the two grouped products and the weighted sum, with the choices given (no routing decision to
     differ in): float32 on the vector units, bfloat16 on the matrix cores where the shape allows."""
@@ -120,20 +121,21 @@ def test_grouped_expert_products_with_given_choices(dtype, width, ff, count, top
         for c in range(top):
             e = int(ids[t, c])
             want[t] += share[t, c].double() * (torch.relu(ups[e] @ x[t]).pow(2) @ downs[e].T)
-    tiles = ops.moe_max_tiles(tokens * top, count)
-    rows = tiles * ops.moe_tile_rows()
+    tile, tiles = ops.moe_tile_rows(tokens * top, count), ops.moe_max_tiles(tokens * top, count)
+    assert tile == (128 if tokens >= 260 else 32)       # steps that bring every expert 128 rows and more use the larger tiles
+    rows = tiles * tile
     sorted_pairs, place = torch.empty(rows, dtype=torch.int32, device="cuda"), torch.empty(tokens * top, dtype=torch.int32, device="cuda")
     tile_expert = torch.empty(tiles, dtype=torch.int32, device="cuda")
     ops.moe_align(ids.cuda(), count, sorted_pairs, place, tile_expert)
     listed = sorted_pairs.cpu()
     assert sorted(listed[listed >= 0].tolist()) == list(range(tokens * top))
-    for tile, e in enumerate(tile_expert.cpu().tolist()):       # every tile holds pairs of its one expert only
-        inside = listed[tile * ops.moe_tile_rows():(tile + 1) * ops.moe_tile_rows()]
+    for number, e in enumerate(tile_expert.cpu().tolist()):       # every tile holds pairs of its one expert only
+        inside = listed[number * tile:(number + 1) * tile]
         assert all(int(ids.view(-1)[p]) == e for p in inside[inside >= 0].tolist()) and (e >= 0 or (inside < 0).all())
     hidden = torch.empty(rows, ff, dtype=dtype, device="cuda")
-    ops.moe_experts(hidden, x.to(dtype).cuda(), torch.stack(ups).to(dtype).cuda(), sorted_pairs, tile_expert, top, gather=True, relu_squared=True)
+    ops.moe_experts(hidden, x.to(dtype).cuda(), torch.stack(ups).to(dtype).cuda(), sorted_pairs, tile_expert, tile, top, gather=True, relu_squared=True)
     outputs = torch.empty(rows, width, dtype=torch.float32, device="cuda")
-    ops.moe_experts(outputs, hidden, torch.stack(downs).to(dtype).cuda(), sorted_pairs, tile_expert, top, gather=False, relu_squared=False)
+    ops.moe_experts(outputs, hidden, torch.stack(downs).to(dtype).cuda(), sorted_pairs, tile_expert, tile, top, gather=False, relu_squared=False)
     got = torch.ones(tokens, width, dtype=torch.float32, device="cuda")
     ops.moe_combine(got, outputs, place, share.cuda(), None)
     close(got - 1.0, want, dtype, f32=2e-5, bf16=1.5e-2)
