@@ -818,7 +818,7 @@ LRS_API int lrs_gather_rows(float* out, const float* x, const int* rows, int n_r
 // residual[r] += w * y[r] * rsqrt(mean(y[r]^2) + eps), all float32: the layer arrangement that normalises what a
 // mixer or feed-forward gives out rather than what it is given.
 template <typename TW>
-__global__ __launch_bounds__(256) void norm_add_kernel(float* __restrict__ residual, const float* __restrict__ y,
+__global__ __launch_bounds__(1024) void norm_add_kernel(float* __restrict__ residual, const float* __restrict__ y,
                                                        const TW* __restrict__ weight, int hidden, float eps) {
   __shared__ float scratch[16];
   const float* src = y + (int64_t)blockIdx.x * hidden;
@@ -832,8 +832,9 @@ __global__ __launch_bounds__(256) void norm_add_kernel(float* __restrict__ resid
 LRS_API int lrs_norm_add(float* residual, const float* y, const void* weight, int w_dtype, int n_rows, int hidden, float eps,
                          void* stream) {
   LRS_REQUIRE(n_rows > 0 && hidden > 0 && eps > 0.f, "norm_add: bad sizes rows=%d hidden=%d", n_rows, hidden);
-  if (w_dtype == LRS_F32) norm_add_kernel<float><<<n_rows, 256, 0, (hipStream_t)stream>>>(residual, y, (const float*)weight, hidden, eps);
-  else if (w_dtype == LRS_BF16) norm_add_kernel<bf16><<<n_rows, 256, 0, (hipStream_t)stream>>>(residual, y, (const bf16*)weight, hidden, eps);
+  const int threads = hidden >= 2048 ? 1024 : 256;       // a wide row alone in a step is a matter of latency: more loads at once
+  if (w_dtype == LRS_F32) norm_add_kernel<float><<<n_rows, threads, 0, (hipStream_t)stream>>>(residual, y, (const float*)weight, hidden, eps);
+  else if (w_dtype == LRS_BF16) norm_add_kernel<bf16><<<n_rows, threads, 0, (hipStream_t)stream>>>(residual, y, (const bf16*)weight, hidden, eps);
   else return lrs_fail("norm_add: unknown weight dtype %d", w_dtype);
   return lrs_check_launch("norm_add");
 }

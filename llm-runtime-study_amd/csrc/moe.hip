@@ -15,6 +15,8 @@
 //                 weight is given, the RMS norm of that sum added into the residual stream.
 #include "common.h"
 
+LRS_API int lrs_compute_units();
+
 namespace {
 
 constexpr int ROUTE_MAX_PER_LANE = 8;     // experts up to 64 * 8
@@ -172,17 +174,20 @@ __global__ __launch_bounds__(256) void moe_experts_kernel(TO* __restrict__ out, 
 // multiplied.
 constexpr int GM = 32, GN = 128, GK = 64, GPAD = 8;
 
-template <typename TO>
+// NT: columns per workgroup, 128 (a wave 32 of them) or 64 (a wave 16: twice the workgroups, for steps of so few rows
+// that 128 columns each would leave compute units without any).
+template <typename TO, int NT>
 __global__ __launch_bounds__(256) void moe_experts_bf16_kernel(TO* __restrict__ out, int ldc, const bf16* __restrict__ a, int lda,
                                                                const bf16* __restrict__ w, int n, int k, const int* __restrict__ sorted,
                                                                const int* __restrict__ tile_expert, int top, int gather, int act) {
   const int expert = tile_expert[blockIdx.x];
   if (expert < 0) return;
   __shared__ __attribute__((aligned(16))) bf16 a_s[GM][GK + GPAD];
-  __shared__ __attribute__((aligned(16))) bf16 b_s[GN][GK + GPAD];
+  __shared__ __attribute__((aligned(16))) bf16 b_s[NT][GK + GPAD];
   __shared__ int row_of[GM];
   const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
-  const int row0 = blockIdx.x * GM, col0 = blockIdx.y * GN;
+  constexpr int WN = NT / 64;                 // products of 16 columns a wave makes side by side
+  const int row0 = blockIdx.x * GM, col0 = blockIdx.y * NT;
   if (tid < GM) {
     const int pair = sorted[row0 + tid];
     row_of[tid] = pair < 0 ? -1 : (gather ? pair / top : row0 + tid);
@@ -194,36 +199,36 @@ __global__ __launch_bounds__(256) void moe_experts_bf16_kernel(TO* __restrict__ 
   const int a_row = tid / 8, a_col = (tid % 8) * 8;
   const int a_src = row_of[a_row];
   const bf16* a_ptr = a_src >= 0 ? a + (int64_t)a_src * lda + a_col : nullptr;
-  bf16x8 a_reg, b_reg[4];
+  bf16x8 a_reg, b_reg[NT / 32];
   const bf16x8 zero = {};
   auto fetch = [&](int k0) {
     a_reg = a_ptr ? *(const bf16x8*)(a_ptr + k0) : zero;
 #pragma unroll
-    for (int p = 0; p < 4; ++p) {
+    for (int p = 0; p < NT / 32; ++p) {
       const int r = p * 32 + a_row;
       b_reg[p] = col0 + r < n ? *(const bf16x8*)(we + (int64_t)(col0 + r) * k + k0 + a_col) : zero;
     }
   };
-  floatx4 acc[2][2] = {};
+  floatx4 acc[2][WN] = {};
   fetch(0);
   const int frag_row = lane % 16, frag_k = (lane / 16) * 8;
   for (int k0 = 0; k0 < k; k0 += GK) {
     *(bf16x8*)&a_s[a_row][a_col] = a_reg;
 #pragma unroll
-    for (int p = 0; p < 4; ++p) *(bf16x8*)&b_s[p * 32 + a_row][a_col] = b_reg[p];
+    for (int p = 0; p < NT / 32; ++p) *(bf16x8*)&b_s[p * 32 + a_row][a_col] = b_reg[p];
     __syncthreads();
     if (k0 + GK < k) fetch(k0 + GK);
 #pragma unroll
     for (int kk = 0; kk < GK; kk += 32) {
-      bf16x8 af[2], bfr[2];
+      bf16x8 af[2], bfr[WN];
 #pragma unroll
       for (int i = 0; i < 2; ++i) af[i] = *(const bf16x8*)&a_s[i * 16 + frag_row][kk + frag_k];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) bfr[i] = *(const bf16x8*)&b_s[wave * 32 + i * 16 + frag_row][kk + frag_k];
+      for (int i = 0; i < WN; ++i) bfr[i] = *(const bf16x8*)&b_s[wave * 16 * WN + i * 16 + frag_row][kk + frag_k];
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int jj = 0; jj < 2; ++jj)
+        for (int jj = 0; jj < WN; ++jj)
           // the weights as the first operand: a lane then holds four consecutive columns of one output row
           acc[i][jj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bfr[jj], af[i], acc[i][jj], 0, 0, 0);
     }
@@ -235,8 +240,8 @@ __global__ __launch_bounds__(256) void moe_experts_bf16_kernel(TO* __restrict__ 
     const int m = i * 16 + lane % 16;
     if (row_of[m] < 0) continue;
 #pragma unroll
-    for (int jj = 0; jj < 2; ++jj) {
-      const int c = col0 + wave * 32 + jj * 16 + (lane / 16) * 4;
+    for (int jj = 0; jj < WN; ++jj) {
+      const int c = col0 + wave * 16 * WN + jj * 16 + (lane / 16) * 4;
 #pragma unroll
       for (int x = 0; x < 4; ++x) {
         if (c + x >= n) continue;
@@ -256,13 +261,18 @@ template <typename TO>
 __global__ __launch_bounds__(256) void moe_experts_bf16_wide_kernel(TO* __restrict__ out, int ldc, const bf16* __restrict__ a, int lda,
                                                                     const bf16* __restrict__ w, int n, int k, const int* __restrict__ sorted,
                                                                     const int* __restrict__ tile_expert, int top, int gather, int act) {
-  const int expert = tile_expert[blockIdx.x];
+  // Workgroups are dealt to the chip's eight dies in turn, each with an L2 of its own: number the tiles so that a die
+  // gets neighbours (row tiles of one expert under one column tile, which share the weights).
+  const int total = gridDim.x * gridDim.y, flat = blockIdx.y * gridDim.x + blockIdx.x;
+  const int logical = total % 8 == 0 ? (flat % 8) * (total / 8) + flat / 8 : flat;
+  const int tile_x = logical % gridDim.x, tile_y = logical / gridDim.x;
+  const int expert = tile_expert[tile_x];
   if (expert < 0) return;
   __shared__ __attribute__((aligned(16))) bf16 a_s[WM][GK + GPAD];
   __shared__ __attribute__((aligned(16))) bf16 b_s[GN][GK + GPAD];
   __shared__ int row_of[WM];
   const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
-  const int row0 = blockIdx.x * WM, col0 = blockIdx.y * GN;
+  const int row0 = tile_x * WM, col0 = tile_y * GN;
   if (tid < WM) {
     const int pair = sorted[row0 + tid];
     row_of[tid] = pair < 0 ? -1 : (gather ? pair / top : row0 + tid);
@@ -331,16 +341,22 @@ __global__ __launch_bounds__(256) void moe_experts_bf16_wide_kernel(TO* __restri
 }
 
 template <typename TW>
-__global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ residual, const float* __restrict__ rows, int hidden,
-                                                          const int* __restrict__ place, const float* __restrict__ weights, int top,
-                                                          const TW* __restrict__ norm_w, float eps) {
-  extern __shared__ float sum[];        // [hidden], then 16 floats for the reduction
+__global__ __launch_bounds__(1024) void moe_combine_kernel(float* __restrict__ residual, const float* __restrict__ rows, int hidden,
+                                                           const int* __restrict__ place, const float* __restrict__ weights, int top,
+                                                           const TW* __restrict__ norm_w, float eps) {
+  extern __shared__ float sum[];        // [hidden], 16 floats for the reduction, then the token's rows and weights [top] each
+  float* share = sum + hidden + 16;
+  int* where = (int*)(share + top);
   const int t = blockIdx.x;
+  for (int c = threadIdx.x; c < top; c += blockDim.x) {
+    share[c] = weights[(int64_t)t * top + c];
+    where[c] = place[(int64_t)t * top + c];
+  }
+  __syncthreads();
   float ss = 0.f;
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
     float acc = 0.f;
-    for (int c = 0; c < top; ++c)
-      acc = fmaf(weights[(int64_t)t * top + c], rows[(int64_t)place[(int64_t)t * top + c] * hidden + i], acc);
+    for (int c = 0; c < top; ++c) acc = fmaf(share[c], rows[(int64_t)where[c] * hidden + i], acc);
     sum[i] = acc;
     ss = fmaf(acc, acc, ss);
   }
@@ -409,13 +425,14 @@ LRS_API int lrs_moe_experts(void* out, int out_dtype, int ldc, const void* a, co
     return lrs_check_launch("moe_experts");
   }
   if (cores) {
-    dim3 grid(max_tiles, (n + GN - 1) / GN);
-    if (out_dtype == LRS_BF16)
-      moe_experts_bf16_kernel<bf16><<<grid, 256, 0, s>>>((bf16*)out, ldc, (const bf16*)a, lda, (const bf16*)w, n, k, sorted, tile_expert, top, gather, act);
-    else if (out_dtype == LRS_F32)
-      moe_experts_bf16_kernel<float><<<grid, 256, 0, s>>>((float*)out, ldc, (const bf16*)a, lda, (const bf16*)w, n, k, sorted, tile_expert, top, gather, act);
-    else
-      return lrs_fail("moe_experts: unknown output dtype %d", out_dtype);
+    // few tiles (single tokens, short portions): 64 columns a workgroup, so that twice as many stream the weights
+    const bool narrow = (int64_t)max_tiles * ((n + GN - 1) / GN) < 4 * lrs_compute_units();
+    dim3 grid(max_tiles, narrow ? (n + 63) / 64 : (n + GN - 1) / GN);
+#define CORES(TO, NT) moe_experts_bf16_kernel<TO, NT><<<grid, 256, 0, s>>>((TO*)out, ldc, (const bf16*)a, lda, (const bf16*)w, n, k, sorted, tile_expert, top, gather, act)
+    if (out_dtype == LRS_BF16) { if (narrow) CORES(bf16, 64); else CORES(bf16, 128); }
+    else if (out_dtype == LRS_F32) { if (narrow) CORES(float, 64); else CORES(float, 128); }
+    else return lrs_fail("moe_experts: unknown output dtype %d", out_dtype);
+#undef CORES
     return lrs_check_launch("moe_experts");
   }
   dim3 grid(max_tiles * (tile / GM), (n + 63) / 64);       // the any-shape form walks a tile of 128 rows as four of 32
@@ -433,12 +450,13 @@ LRS_API int lrs_moe_combine(float* residual, const float* rows, int tokens, int 
                             int top, const void* norm_w, int norm_dtype, float eps, void* stream) {
   LRS_REQUIRE(tokens > 0 && hidden > 0 && top > 0, "moe_combine: bad sizes tokens=%d hidden=%d top=%d", tokens, hidden, top);
   LRS_REQUIRE(!norm_w || eps > 0.f, "moe_combine: eps must be positive");
-  const size_t lds = (size_t)(hidden + 16) * sizeof(float);
-  LRS_REQUIRE(lds <= 64 * 1024, "moe_combine: a width of %d is too much", hidden);
+  const size_t lds = (size_t)(hidden + 16 + 2 * top) * sizeof(float);
+  LRS_REQUIRE(lds <= 64 * 1024, "moe_combine: a width of %d with %d choices is too much", hidden, top);
   hipStream_t s = (hipStream_t)stream;
+  const int threads = hidden >= 2048 ? 1024 : 256;
   if (norm_w && norm_dtype == LRS_BF16)
-    moe_combine_kernel<bf16><<<tokens, 256, lds, s>>>(residual, rows, hidden, place, weights, top, (const bf16*)norm_w, eps);
+    moe_combine_kernel<bf16><<<tokens, threads, lds, s>>>(residual, rows, hidden, place, weights, top, (const bf16*)norm_w, eps);
   else
-    moe_combine_kernel<float><<<tokens, 256, lds, s>>>(residual, rows, hidden, place, weights, top, (const float*)norm_w, eps);
+    moe_combine_kernel<float><<<tokens, threads, lds, s>>>(residual, rows, hidden, place, weights, top, (const float*)norm_w, eps);
   return lrs_check_launch("moe_combine");
 }
