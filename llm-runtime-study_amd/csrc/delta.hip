@@ -217,6 +217,56 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(const float* __restrict
   }
 }
 
+// The same for steps in which every request brings one token: nothing is staged, a thread reads its slices of the key
+// and the query where the preparation left them, and as many workgroups as fit run side by side (no LDS holds them back).
+template <int ROWS>
+__global__ __launch_bounds__(256) void delta_scan_single_kernel(const float* __restrict__ qkv, const float* __restrict__ gates,
+                                                                const int* __restrict__ slot_ids, float* __restrict__ state,
+                                                                int64_t state_stride, int G, int H, int d, int dv, float* __restrict__ raw_out) {
+  const int r = blockIdx.x, h = blockIdx.y, block = blockIdx.z, tid = threadIdx.x;
+  const int channels = 2 * G * d + H * dv, hk = h / (H / G);
+  const int c = tid / SPLIT, s = tid % SPLIT, column = block * COLUMNS + c;
+  if (column >= dv) return;
+  float* st = state + (int64_t)slot_ids[r] * state_stride + (int64_t)h * ROWS * dv * SPLIT + (int64_t)block * COLUMNS * SPLIT;
+  const float* row = qkv + (int64_t)r * channels;
+  float S[ROWS], kk[ROWS], qq[ROWS];
+#pragma unroll
+  for (int i = 0; i < ROWS; ++i) S[i] = st[(int64_t)i * dv * SPLIT + tid];
+  if (d % 4 == 0 && channels % 4 == 0) {          // every piece of four values is 16 bytes aligned
+#pragma unroll
+    for (int p = 0; p < ROWS / 4; ++p) {
+      const int at = s * ROWS + 4 * p;
+      const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+      const float4 a = at < d ? *(const float4*)(row + hk * d + at) : zero, b = at < d ? *(const float4*)(row + G * d + hk * d + at) : zero;
+      qq[4 * p] = a.x, qq[4 * p + 1] = a.y, qq[4 * p + 2] = a.z, qq[4 * p + 3] = a.w;
+      kk[4 * p] = b.x, kk[4 * p + 1] = b.y, kk[4 * p + 2] = b.z, kk[4 * p + 3] = b.w;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i) {
+      const int at = s * ROWS + i;
+      qq[i] = at < d ? row[hk * d + at] : 0.f;
+      kk[i] = at < d ? row[G * d + hk * d + at] : 0.f;
+    }
+  }
+  const float v = row[2 * G * d + h * dv + column];
+  const float beta = gates[(int64_t)r * 2 * H + h], g = gates[(int64_t)r * 2 * H + H + h];
+  float dk = 0.f, dq = 0.f, kq = 0.f;
+#pragma unroll
+  for (int i = 0; i < ROWS; ++i) {
+    dk = fmaf(S[i], kk[i], dk);
+    dq = fmaf(S[i], qq[i], dq);
+    kq = fmaf(kk[i], qq[i], kq);
+  }
+  dk = row_sum16(dk);
+  dq = row_sum16(dq);
+  kq = row_sum16(kq);
+  const float u = beta * (v - g * dk);
+#pragma unroll
+  for (int i = 0; i < ROWS; ++i) st[(int64_t)i * dv * SPLIT + tid] = fmaf(kk[i], u, g * S[i]);
+  if (s == 0) raw_out[(int64_t)r * H * dv + h * dv + column] = fmaf(u, kq, g * dq);
+}
+
 // The head's read-out divided by its root mean square over vdim, times the norm's weight, times silu(gate): a wave a
 // (token, head).
 template <typename TP, typename TO>
@@ -272,7 +322,11 @@ LRS_API int lrs_delta_rule(void* out, int out_dtype, const void* proj, int proj_
     if (taps > 1)                                                                                                             \
       delta_conv_keep_kernel<TP><<<kgrid, 256, 0, s>>>((const TP*)proj, ld, cu, slot_ids, state, state_stride, conv_offset,  \
                                                        taps, channels);                                                       \
-    if (rows == 4) delta_scan_kernel<4, 16><<<sgrid, 256, lds, s>>>(qkv, gates, cu, slot_ids, state, state_stride, G, H, d, dv, raw);       \
+    if (tokens == requests) {        /* one token each: token r is request r's */                                             \
+      if (rows == 4) delta_scan_single_kernel<4><<<sgrid, 256, 0, s>>>(qkv, gates, slot_ids, state, state_stride, G, H, d, dv, raw);        \
+      else if (rows == 8) delta_scan_single_kernel<8><<<sgrid, 256, 0, s>>>(qkv, gates, slot_ids, state, state_stride, G, H, d, dv, raw);   \
+      else delta_scan_single_kernel<16><<<sgrid, 256, 0, s>>>(qkv, gates, slot_ids, state, state_stride, G, H, d, dv, raw);                 \
+    } else if (rows == 4) delta_scan_kernel<4, 16><<<sgrid, 256, lds, s>>>(qkv, gates, cu, slot_ids, state, state_stride, G, H, d, dv, raw);       \
     else if (rows == 8) delta_scan_kernel<8, 16><<<sgrid, 256, lds, s>>>(qkv, gates, cu, slot_ids, state, state_stride, G, H, d, dv, raw);  \
     else delta_scan_kernel<16, 8><<<sgrid, 256, lds, s>>>(qkv, gates, cu, slot_ids, state, state_stride, G, H, d, dv, raw);                 \
     delta_gate_kernel<TP, TO><<<(unsigned)((pairs + 3) / 4), 256, 0, s>>>(raw, (const TP*)proj, ld, gate_at, norm_w, eps, tokens, H, dv, (TO*)out); \
