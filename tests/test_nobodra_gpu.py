@@ -371,3 +371,40 @@ def test_greedy_generation_through_engine_and_scheduler(models):
     engine = Engine.from_model_dir(folder, dtype="float32", max_seq_len=128, max_batch_size=2, max_num_batched_tokens=16)
     assert engine.generate_tokens(prompts, max_new_tokens=6) == want
     assert engine.cache_manager.active_requests == 0
+
+
+def test_command_line_and_trace_run_as_programs(models, tmp_path):
+    """The two programs, each a process of its own, find the architecture by the folder's config.json: greedy tokens from the
+    command line (token ids in, token ids out, random weights from a seed as well), and a mixed replay through bin/trace_run."""
+    import os
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    root = Path(__file__).resolve().parents[1]
+    env = dict(os.environ, PYTHONPATH=str(root))
+    folder, raw, requests, want = models["routed"]
+    _, weights = plain.load_model_dir(folder)
+    prompt = requests["routed2"]
+    ids = list(prompt)
+    for _ in range(5):
+        ids.append(int(plain.forward(weights, raw, ids)[-1].argmax()))
+    proc = subprocess.run([sys.executable, "-m", "llm_runtime_study_amd", "--model", str(folder), "--prompt-ids", ",".join(map(str, prompt)),
+                           "--max-new-tokens", "5", "--dtype", "float32", "--max-seq-len", "64", "--no-metrics"],
+                          capture_output=True, text=True, timeout=300, env=env, cwd=tmp_path)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [int(t) for t in proc.stdout.split()] == ids[len(prompt):]
+    only_config = tmp_path / "only_config"
+    only_config.mkdir()
+    (only_config / "config.json").write_text((folder / "config.json").read_text())
+    proc = subprocess.run([sys.executable, "-m", "llm_runtime_study_amd", "--model", str(only_config), "--random-weights", "3", "--prompt-ids", "1,2,3",
+                           "--max-new-tokens", "4", "--max-seq-len", "64", "--no-metrics"], capture_output=True, text=True, timeout=300, env=env, cwd=tmp_path)
+    assert proc.returncode == 0 and len(proc.stdout.split()) == 4, proc.stderr[-2000:]
+    few = dict(list(requests.items())[2:6])
+    steps, peak = traces.mixed(few, seed=9, max_live=3)
+    out = tmp_path / "replayed"
+    proc = subprocess.run([sys.executable, str(root / "bin" / "trace_run"), "--model", str(folder), "--dtype", "float32", "--out", str(out),
+                           "--max-tokens", str(peak)], input=traces.strip(steps), capture_output=True, text=True, timeout=300, env=env, cwd=tmp_path)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [line for line in proc.stdout.splitlines() if line.startswith("done ")] == [f"done {s['step']}" for s in steps]
+    compare(traces.collect(steps, out, raw["vocab"]), want, "float32")
