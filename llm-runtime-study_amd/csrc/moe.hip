@@ -340,6 +340,117 @@ __global__ __launch_bounds__(256) void moe_experts_bf16_wide_kernel(TO* __restri
   }
 }
 
+// The grouped product for large steps the way this package's many-rows product is made (gemm_bf16_wide in gemm.hip):
+// 128 sorted rows x 256 columns of one expert per workgroup of four waves, a wave 64 rows x 128 columns; memory writes
+// slices of 32 of K straight into LDS (fetch_to_lds), three stages, in a layout whose rows swap places and whose chunks
+// are turned round by the row number so that every fragment read touches every bank once; no registers hold a slice on
+// its way.  What differs from the dense kernel: a row's address comes from the sorted list (the token of the pair, or
+// the sorted row itself), the weights are the tile's expert's, rows that pad an expert's run are fetched from the tile's
+// first row and never written, and the epilogue may square the positive part.
+template <typename TO>
+__global__ __launch_bounds__(256, 2) void moe_experts_bf16_fetch_kernel(TO* __restrict__ out, int ldc, const bf16* __restrict__ x, int lda,
+                                                                        const bf16* __restrict__ w, int n, int k, const int* __restrict__ sorted,
+                                                                        const int* __restrict__ tile_expert, int tiles_m, int tiles_n, int top,
+                                                                        int gather, int act) {
+  constexpr int BM = 128, BN = 256, BK = 32, STAGES = 3;
+  constexpr int XL = BM / 16 / 4, WL = BN / 16 / 4;
+  constexpr int STAGE_ELEMENTS = (BM + BN) * BK;
+  __shared__ __attribute__((aligned(64))) bf16 slices[STAGES * STAGE_ELEMENTS];
+  const int tid = threadIdx.x, lane = tid % WAVE, wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
+  const int r = lane & 15, g = lane >> 4;
+  int id = blockIdx.x;
+  const int tiles = tiles_m * tiles_n;
+  if (tiles % 8 == 0) id = (id % 8) * (tiles / 8) + id / 8;        // consecutive workgroups go to different dies
+  const int band = id / (4 * tiles_n), within = id % (4 * tiles_n);
+  const int band_rows = tiles_m - band * 4 < 4 ? tiles_m - band * 4 : 4;
+  const int tile_m = band * 4 + within % band_rows;
+  const int expert = tile_expert[tile_m];
+  if (expert < 0) return;
+  const int m0 = tile_m * BM, n0 = (within / band_rows) * BN;
+  const bf16* we = w + (int64_t)expert * n * k;
+  const int wm = (wave >> 1) * 64, wn = (wave & 1) * 128;
+  const int place_row = (lane >> 2) ^ ((lane >> 5) & 1);
+  const int place_chunk = (lane & 3) ^ ((place_row >> 1) & 3);
+  const int first_pair = sorted[m0];                                 // a tile in use begins with a row in use
+  const int fallback = gather ? first_pair / top : m0;
+  unsigned xoff[XL], woff[WL];
+#pragma unroll
+  for (int i = 0; i < XL; ++i) {
+    const int at = m0 + 16 * (wave + 4 * i) + place_row, pair = sorted[at];
+    const int row = pair < 0 ? fallback : (gather ? pair / top : at);
+    xoff[i] = (unsigned)((row * lda + place_chunk * 8) * 2);
+  }
+#pragma unroll
+  for (int i = 0; i < WL; ++i) {
+    const int row = n0 + 16 * (wave + 4 * i) + place_row;
+    woff[i] = (unsigned)(((row < n ? row : n - 1) * k + place_chunk * 8) * 2);
+  }
+  const int frag = ((r ^ ((r >> 3) & 1)) * 4 + (g ^ ((r >> 1) & 3))) * 8;
+  floatx4 acc[8][4];
+#pragma unroll
+  for (int it = 0; it < 8; ++it)
+#pragma unroll
+    for (int jt = 0; jt < 4; ++jt) acc[it][jt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  const int steps = k / BK;
+  const unsigned slices_address = (unsigned)(uintptr_t)(__attribute__((address_space(3))) bf16*)slices;
+  auto fetch = [&](int kt, int stage) {
+    const int at = (kt < steps ? kt : steps - 1) * BK * 2;
+    const unsigned to = slices_address + (unsigned)(stage * STAGE_ELEMENTS * 2 + wave * 1024);
+#pragma unroll
+    for (int i = 0; i < XL; ++i) fetch_to_lds((const char*)x + at, xoff[i], to + (unsigned)(i * 4096));
+#pragma unroll
+    for (int i = 0; i < WL; ++i) fetch_to_lds((const char*)we + at, woff[i], to + (unsigned)(BM * BK * 2 + i * 4096));
+  };
+  auto multiply = [&](int stage) {
+    const bf16* xs = slices + stage * STAGE_ELEMENTS;
+    const bf16* ws = xs + BM * BK;
+    bf16x8 xf[4];
+#pragma unroll
+    for (int jt = 0; jt < 4; ++jt) xf[jt] = *(const bf16x8*)(xs + frag + (wm + jt * 16) * BK);
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+      const bf16x8 wf = *(const bf16x8*)(ws + frag + (wn + it * 16) * BK);
+#pragma unroll
+      for (int jt = 0; jt < 4; ++jt) acc[it][jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf[jt], acc[it][jt], 0, 0, 0);
+    }
+  };
+  int m0_opaque = m0;
+  fetch(0, 0);
+  fetch(1, 1);
+  fetched_then_barrier<6>();
+  int stage = 0;
+  for (int kt = 0; kt < steps; ++kt) {
+    fetch(kt + 2, stage == 0 ? 2 : stage - 1);
+    multiply(stage);
+    fetched_then_barrier<6>();
+    stage = stage == STAGES - 1 ? 0 : stage + 1;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");               // the fetches past K that nobody reads
+  asm volatile("" : "+s"(ldc), "+s"(m0_opaque));
+#pragma unroll
+  for (int jt = 0; jt < 4; ++jt) {
+    const int at = m0_opaque + wm + jt * 16 + r;
+    const bool in_use = sorted[at] >= 0;
+    const int64_t row_at = (int64_t)at * ldc;
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+      const int row0 = n0 + wn + it * 16 + 4 * g;                  // this lane's four weight rows = output columns
+      if (in_use && row0 < n) {
+        floatx4 v = acc[it][jt];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = __shfl(v[i], lane, WAVE);      // keeps the loop above free of spills, as in the dense kernel
+        if (act == ACT_RELU_SQUARED) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v[i] = v[i] > 0.f ? v[i] * v[i] : 0.f;
+        }
+        if constexpr (sizeof(TO) == 2) *(bf16x4*)((bf16*)out + row_at + row0) = bf16x4{(bf16)v[0], (bf16)v[1], (bf16)v[2], (bf16)v[3]};
+        else *(floatx4*)((float*)out + row_at + row0) = v;
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+}
+
 template <typename TW>
 __global__ __launch_bounds__(1024) void moe_combine_kernel(float* __restrict__ residual, const float* __restrict__ rows, int hidden,
                                                            const int* __restrict__ place, const float* __restrict__ weights, int top,
@@ -372,9 +483,12 @@ __global__ __launch_bounds__(1024) void moe_combine_kernel(float* __restrict__ r
 
 }  // namespace
 
-// Rows of a tile of the grouped products: 32, or 128 once the step brings every expert 128 rows and more on average
-// (follows from the step's shape alone, so that recorded and captured steps keep it).
-LRS_API int lrs_moe_tile_rows(int pairs, int experts) { return (int64_t)pairs >= (int64_t)WM * experts ? WM : GM; }
+// Rows of a tile of the grouped products: 32, or 128 once the step brings every expert 48 rows and more on average: what
+// a step of a few dozen rows an expert pays for is how often an expert's weights are fetched, once a tile, and not
+// the matrix instructions on rows that only pad (8 layers at the 8B sizes, a prompt of 512 tokens, 128 rows an expert:
+// 6.9 ms with tiles of 128, 9.8 ms with tiles of 32).  Follows from the step's shape alone, so that recorded and captured
+// steps keep it.
+LRS_API int lrs_moe_tile_rows(int pairs, int experts) { return (int64_t)pairs >= (int64_t)48 * experts ? WM : GM; }
 
 // The most tiles that `pairs` (token, choice) pairs of `experts` experts can fill: every expert in use ends in at
 // most one tile that is not full.
@@ -414,6 +528,20 @@ LRS_API int lrs_moe_experts(void* out, int out_dtype, int ldc, const void* a, co
   LRS_REQUIRE(act == ACT_NONE || act == ACT_RELU_SQUARED, "moe_experts: unknown activation %d", act);
   hipStream_t s = (hipStream_t)stream;
   const bool cores = dtype == LRS_BF16 && k % GK == 0 && lda % 8 == 0 && ((uintptr_t)a % 16) == 0 && ((uintptr_t)w % 16) == 0;
+  // large steps of shapes the fetching kernel takes: whole slices of 32 of K, rows of the output 16 bytes aligned, offsets
+  // that fit 32 bits
+  const bool fetching = cores && tile == WM && k % 32 == 0 && n % 4 == 0 && ldc % 4 == 0 && ((uintptr_t)out % 16) == 0 && k >= 64 &&
+                        (int64_t)n * k < (1ll << 30) && (gather ? (int64_t)max_tiles * tile / top + 1 : (int64_t)max_tiles * tile) * lda < (1ll << 30);
+  if (fetching) {
+    const int tiles_n = (n + 255) / 256;
+    if (out_dtype == LRS_BF16)
+      moe_experts_bf16_fetch_kernel<bf16><<<max_tiles * tiles_n, 256, 0, s>>>((bf16*)out, ldc, (const bf16*)a, lda, (const bf16*)w, n, k, sorted, tile_expert, max_tiles, tiles_n, top, gather, act);
+    else if (out_dtype == LRS_F32)
+      moe_experts_bf16_fetch_kernel<float><<<max_tiles * tiles_n, 256, 0, s>>>((float*)out, ldc, (const bf16*)a, lda, (const bf16*)w, n, k, sorted, tile_expert, max_tiles, tiles_n, top, gather, act);
+    else
+      return lrs_fail("moe_experts: unknown output dtype %d", out_dtype);
+    return lrs_check_launch("moe_experts");
+  }
   if (cores && tile == WM) {
     dim3 grid(max_tiles, (n + GN - 1) / GN);
     if (out_dtype == LRS_BF16)

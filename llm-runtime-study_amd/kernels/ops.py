@@ -1165,8 +1165,8 @@ def delta_rule(out: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, token
 # ------------------------------------------------------------------- routed experts
 def moe_tile_rows(pairs: int, experts: int) -> int:
     """Rows of a tile of the grouped products for a step of `pairs` (token, choice) pairs: 32, or 128 once every expert
-    gets 128 rows and more on average."""
-    return 128 if pairs >= 128 * experts else 32
+    gets 48 rows and more on average (see csrc/moe.hip)."""
+    return 128 if pairs >= 48 * experts else 32
 
 
 def moe_max_tiles(pairs: int, experts: int) -> int:

@@ -105,7 +105,7 @@ def moe_weights(width, ff, count, seed):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("width,ff,count,top,tokens", [(64, 48, 6, 2, 50), (128, 64, 70, 3, 200), (128, 128, 8, 8, 33), (40, 24, 5, 1, 7), (192, 64, 16, 4, 1),
-                                                       (128, 192, 3, 2, 300), (72, 40, 2, 2, 260)])
+                                                       (128, 192, 3, 2, 400), (72, 40, 2, 2, 260), (256, 320, 4, 2, 600), (512, 96, 2, 1, 700)])
 def test_grouped_expert_products_with_given_choices(dtype, width, ff, count, top, tokens):
     """The sort by expert, the two grouped products and the weighted sum, with the choices given (no routing decision to
     differ in): float32 on the vector units, bfloat16 on the matrix cores where the shape allows."""
@@ -122,7 +122,7 @@ def test_grouped_expert_products_with_given_choices(dtype, width, ff, count, top
             e = int(ids[t, c])
             want[t] += share[t, c].double() * (torch.relu(ups[e] @ x[t]).pow(2) @ downs[e].T)
     tile, tiles = ops.moe_tile_rows(tokens * top, count), ops.moe_max_tiles(tokens * top, count)
-    assert tile == (128 if tokens >= 260 else 32)       # steps that bring every expert 128 rows and more use the larger tiles
+    assert tile == (128 if tokens >= 260 else 32)       # steps that bring every expert 48 rows and more use the larger tiles
     rows = tiles * tile
     sorted_pairs, place = torch.empty(rows, dtype=torch.int32, device="cuda"), torch.empty(tokens * top, dtype=torch.int32, device="cuda")
     tile_expert = torch.empty(tiles, dtype=torch.int32, device="cuda")
