@@ -816,10 +816,11 @@ LRS_API int lrs_gather_rows(float* out, const float* x, const int* rows, int n_r
 
 // ------------------------------------------------ norm of a sublayer's output, added to the stream
 // residual[r] += w * y[r] * rsqrt(mean(y[r]^2) + eps), all float32: the layer arrangement that normalises what a
-// mixer or feed-forward gives out rather than what it is given.
+// mixer or feed-forward gives out rather than what it is given.  With `rounded` the updated row is also left in
+// bfloat16, for the sublayer that reads the stream next (no kernel of its own for that).
 template <typename TW>
 __global__ __launch_bounds__(1024) void norm_add_kernel(float* __restrict__ residual, const float* __restrict__ y,
-                                                       const TW* __restrict__ weight, int hidden, float eps) {
+                                                       const TW* __restrict__ weight, int hidden, float eps, bf16* __restrict__ rounded) {
   __shared__ float scratch[16];
   const float* src = y + (int64_t)blockIdx.x * hidden;
   float* dst = residual + (int64_t)blockIdx.x * hidden;
@@ -827,14 +828,18 @@ __global__ __launch_bounds__(1024) void norm_add_kernel(float* __restrict__ resi
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) ss = fmaf(src[i], src[i], ss);
   ss = block_sum(ss, scratch);
   const float inv = 1.0f / sqrtf(ss / (float)hidden + eps);
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] += to_float(weight[i]) * (src[i] * inv);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float v = dst[i] + to_float(weight[i]) * (src[i] * inv);
+    dst[i] = v;
+    if (rounded) rounded[(int64_t)blockIdx.x * hidden + i] = (bf16)v;
+  }
 }
 LRS_API int lrs_norm_add(float* residual, const float* y, const void* weight, int w_dtype, int n_rows, int hidden, float eps,
-                         void* stream) {
+                         void* rounded, void* stream) {
   LRS_REQUIRE(n_rows > 0 && hidden > 0 && eps > 0.f, "norm_add: bad sizes rows=%d hidden=%d", n_rows, hidden);
   const int threads = hidden >= 2048 ? 1024 : 256;       // a wide row alone in a step is a matter of latency: more loads at once
-  if (w_dtype == LRS_F32) norm_add_kernel<float><<<n_rows, threads, 0, (hipStream_t)stream>>>(residual, y, (const float*)weight, hidden, eps);
-  else if (w_dtype == LRS_BF16) norm_add_kernel<bf16><<<n_rows, threads, 0, (hipStream_t)stream>>>(residual, y, (const bf16*)weight, hidden, eps);
+  if (w_dtype == LRS_F32) norm_add_kernel<float><<<n_rows, threads, 0, (hipStream_t)stream>>>(residual, y, (const float*)weight, hidden, eps, (bf16*)rounded);
+  else if (w_dtype == LRS_BF16) norm_add_kernel<bf16><<<n_rows, threads, 0, (hipStream_t)stream>>>(residual, y, (const bf16*)weight, hidden, eps, (bf16*)rounded);
   else return lrs_fail("norm_add: unknown weight dtype %d", w_dtype);
   return lrs_check_launch("norm_add");
 }

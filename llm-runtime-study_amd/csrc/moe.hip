@@ -454,7 +454,7 @@ __global__ __launch_bounds__(256, 2) void moe_experts_bf16_fetch_kernel(TO* __re
 template <typename TW>
 __global__ __launch_bounds__(1024) void moe_combine_kernel(float* __restrict__ residual, const float* __restrict__ rows, int hidden,
                                                            const int* __restrict__ place, const float* __restrict__ weights, int top,
-                                                           const TW* __restrict__ norm_w, float eps) {
+                                                           const TW* __restrict__ norm_w, float eps, bf16* __restrict__ rounded) {
   extern __shared__ float sum[];        // [hidden], 16 floats for the reduction, then the token's rows and weights [top] each
   float* share = sum + hidden + 16;
   int* where = (int*)(share + top);
@@ -472,13 +472,16 @@ __global__ __launch_bounds__(1024) void moe_combine_kernel(float* __restrict__ r
     ss = fmaf(acc, acc, ss);
   }
   float* out = residual + (int64_t)t * hidden;
-  if (!norm_w) {
-    for (int i = threadIdx.x; i < hidden; i += blockDim.x) out[i] += sum[i];
-    return;
+  float inv = 1.f;
+  if (norm_w) {
+    ss = block_sum(ss, sum + hidden);
+    inv = 1.0f / sqrtf(ss / (float)hidden + eps);
   }
-  ss = block_sum(ss, sum + hidden);
-  const float inv = 1.0f / sqrtf(ss / (float)hidden + eps);
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) out[i] += sum[i] * inv * to_float(norm_w[i]);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float v = out[i] + (norm_w ? sum[i] * inv * to_float(norm_w[i]) : sum[i]);
+    out[i] = v;
+    if (rounded) rounded[(int64_t)t * hidden + i] = (bf16)v;       // the stream as the next sublayer reads it
+  }
 }
 
 }  // namespace
@@ -573,9 +576,10 @@ LRS_API int lrs_moe_experts(void* out, int out_dtype, int ldc, const void* a, co
   return lrs_check_launch("moe_experts");
 }
 
-// residual [tokens, hidden] += (norm of) sum_c weights[t, c] * rows[place[t, c]]; norm_w null: the plain sum.
+// residual [tokens, hidden] += (norm of) sum_c weights[t, c] * rows[place[t, c]]; norm_w null: the plain sum; rounded:
+// where the updated rows are left in bfloat16 as well, or null.
 LRS_API int lrs_moe_combine(float* residual, const float* rows, int tokens, int hidden, const int* place, const float* weights,
-                            int top, const void* norm_w, int norm_dtype, float eps, void* stream) {
+                            int top, const void* norm_w, int norm_dtype, float eps, void* rounded, void* stream) {
   LRS_REQUIRE(tokens > 0 && hidden > 0 && top > 0, "moe_combine: bad sizes tokens=%d hidden=%d top=%d", tokens, hidden, top);
   LRS_REQUIRE(!norm_w || eps > 0.f, "moe_combine: eps must be positive");
   const size_t lds = (size_t)(hidden + 16 + 2 * top) * sizeof(float);
@@ -583,8 +587,8 @@ LRS_API int lrs_moe_combine(float* residual, const float* rows, int tokens, int 
   hipStream_t s = (hipStream_t)stream;
   const int threads = hidden >= 2048 ? 1024 : 256;
   if (norm_w && norm_dtype == LRS_BF16)
-    moe_combine_kernel<bf16><<<tokens, threads, lds, s>>>(residual, rows, hidden, place, weights, top, (const bf16*)norm_w, eps);
+    moe_combine_kernel<bf16><<<tokens, threads, lds, s>>>(residual, rows, hidden, place, weights, top, (const bf16*)norm_w, eps, (bf16*)rounded);
   else
-    moe_combine_kernel<float><<<tokens, threads, lds, s>>>(residual, rows, hidden, place, weights, top, (const float*)norm_w, eps);
+    moe_combine_kernel<float><<<tokens, threads, lds, s>>>(residual, rows, hidden, place, weights, top, (const float*)norm_w, eps, (bf16*)rounded);
   return lrs_check_launch("moe_combine");
 }

@@ -145,7 +145,7 @@ _SIGNATURES = {
     "lrs_choose_tokens_static_max_parts": (c_int, []),
     "lrs_filter_logits": (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "lrs_round_rows": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_void_p]),
-    "lrs_norm_add": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_void_p]),
+    "lrs_norm_add": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_void_p, c_void_p]),
     "lrs_delta_state_rows": (c_int, [c_int]),
     "lrs_delta_rule": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
                                c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p]),
@@ -155,7 +155,7 @@ _SIGNATURES = {
     "lrs_moe_align": (c_int, [c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p]),
     "lrs_moe_experts": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
                                 c_int, c_int, c_void_p]),
-    "lrs_moe_combine": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_float, c_void_p]),
+    "lrs_moe_combine": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p]),
 }
 
 
@@ -438,13 +438,22 @@ def round_rows(out: torch.Tensor, x: torch.Tensor) -> None:
     _launch("lrs_round_rows", _dev(out, "out"), dtype_code(out.dtype), _dev(x, "x"), x.numel(), _stream())
 
 
-def norm_add(residual: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float) -> None:
-    """residual += weight * y * rsqrt(mean(y^2) + eps), row by row, in float32: the norm of a sublayer's output added to the stream."""
+def _rounded(rounded: torch.Tensor | None, rows: int, hidden: int, who: str):
+    if rounded is None:
+        return None
+    _need(rounded.dtype == torch.bfloat16 and rounded.is_contiguous() and rounded.shape == (rows, hidden), f"{who}: the rounded rows must be contiguous bfloat16 [T, H]")
+    return _dev(rounded, "rounded")
+
+
+def norm_add(residual: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float, rounded: torch.Tensor | None = None) -> None:
+    """residual += weight * y * rsqrt(mean(y^2) + eps), row by row, in float32: the norm of a sublayer's output added to the
+    stream.  rounded: bfloat16 [T, H] that receives the updated rows as well."""
     n_rows, hidden = y.shape
     _need(residual.dtype == torch.float32 and y.dtype == torch.float32 and residual.is_contiguous() and y.is_contiguous()
           and residual.shape[0] >= n_rows and residual.shape[1] == hidden, "norm_add: residual and y must be contiguous float32 [T, H]")
     _need(weight.is_contiguous() and weight.numel() == hidden, f"norm_add: weight must hold {hidden} values")
-    _launch("lrs_norm_add", _dev(residual, "residual"), _dev(y, "y"), _dev(weight, "weight"), dtype_code(weight.dtype), n_rows, hidden, eps, _stream())
+    _launch("lrs_norm_add", _dev(residual, "residual"), _dev(y, "y"), _dev(weight, "weight"), dtype_code(weight.dtype), n_rows, hidden, eps,
+            _rounded(rounded, n_rows, hidden, "norm_add"), _stream())
 
 
 def rope_table(cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor) -> None:
@@ -1217,9 +1226,10 @@ def moe_experts(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, sorted_pair
 
 
 def moe_combine(residual: torch.Tensor, rows: torch.Tensor, place: torch.Tensor, weights: torch.Tensor, norm_weight: torch.Tensor | None,
-                eps: float = 0.0) -> None:
+                eps: float = 0.0, rounded: torch.Tensor | None = None) -> None:
     """residual [T, H] += sum over a token's choices of weights[t, c] * rows[place[t, c]]; with norm_weight: the RMS
-    norm (weight norm_weight, eps) of that sum instead of the sum itself."""
+    norm (weight norm_weight, eps) of that sum instead of the sum itself.  rounded: bfloat16 [T, H] that receives the
+    updated rows as well."""
     tokens, top = weights.shape
     hidden = rows.shape[1]
     _need(residual.dtype == torch.float32 and residual.is_contiguous() and residual.shape[0] >= tokens and residual.shape[1] == hidden
@@ -1228,4 +1238,5 @@ def moe_combine(residual: torch.Tensor, rows: torch.Tensor, place: torch.Tensor,
           and weights.is_contiguous(), "moe_combine: place must be int32 [T * top] and weights float32 [T, top]")
     _need(norm_weight is None or (norm_weight.numel() == hidden and norm_weight.is_contiguous()), "moe_combine: norm weight must hold H values")
     _launch("lrs_moe_combine", _dev(residual, "residual"), _dev(rows, "rows"), tokens, hidden, _dev(place, "place"), _dev(weights, "weights"), top,
-            None if norm_weight is None else _dev(norm_weight, "norm_weight"), 0 if norm_weight is None else dtype_code(norm_weight.dtype), eps, _stream())
+            None if norm_weight is None else _dev(norm_weight, "norm_weight"), 0 if norm_weight is None else dtype_code(norm_weight.dtype), eps,
+            _rounded(rounded, tokens, hidden, "moe_combine"), _stream())

@@ -118,8 +118,15 @@ class DecoderModel:
             self.after_embedding.forward(ctx, h)
         schedule = self.spec.schedule
         begun = None   # the next layer's first norm, if the product that last updated h began it
+        handed = handed_kind = None   # what the layer before hands the next one of its kind (a block's `handover_kind`)
         for position, entry in enumerate(schedule):
             layer = self.layers[entry.layer]
+            kind = getattr(layer, "handover_kind", None)
+            if kind is not None:
+                handed = layer.forward(ctx, h, ctx.layer_cache(position), given=handed if handed_kind == kind else None)
+                handed_kind, begun = kind, None
+                continue
+            handed = handed_kind = None
             if not getattr(layer, "chains_norms", False):
                 layer.forward(ctx, h, ctx.layer_cache(position))
                 begun = None

@@ -32,6 +32,10 @@ Optional, each announced by a class attribute (a part without it is simply given
                               normalised input a previous block began and may return the next one;
                               `first_norm` is the norm it applies to its input
 
+  handover_kind = "..."       block: forward(ctx, h, cache, given=None) returns something for the next block to start from
+                              (the stream already rounded to the activation dtype, say), which the model passes on as
+                              `given` to the block that runs next if that one names the same kind, and to no other
+
   wants_query_groups = True   mixer (a block passes it on): the step function cuts the tokens of a ragged step into
                               query groups for it: ctx.qblock_token0 / ctx.qblock_count [ctx.num_qblocks] list groups of
                               at most ctx.max_qblock consecutive tokens of one request, longest context first, which

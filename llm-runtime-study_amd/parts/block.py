@@ -145,6 +145,10 @@ class OutputNormBlock(Part):
     def wants_query_groups(self) -> bool:
         return getattr(self.mixer, "wants_query_groups", False)
 
+    # What a block of this kind hands the next one of its kind (models/decoder.py passes it on as `given`): the stream
+    # rounded to bfloat16, left by the kernel that last added into it, so that no kernel of its own rounds it again.
+    handover_kind = "rounded_stream"
+
     @staticmethod
     def _input(ctx, h):
         """The stream as the activation a sublayer reads: itself in float32 runs, else rounded once."""
@@ -160,24 +164,39 @@ class OutputNormBlock(Part):
         ops.fill_i32(y.view(torch.int32), 0)
         return y
 
-    def forward(self, ctx, h, cache):
-        x = self._input(ctx, h)
+    def _add_normed(self, ctx, norm, h, y, name):
+        """h += norm(y); returns the updated stream as the next reader's activation if the norm's kernel left it (bfloat16
+        runs with a norm that can), else None."""
+        if ctx.dtype == torch.bfloat16 and getattr(norm, "rounds_stream", False):
+            rounded = ctx.scratch(name, tuple(h.shape), torch.bfloat16)
+            norm.add_normed(ctx, h, y, rounded=rounded)
+            return rounded
+        norm.add_normed(ctx, h, y)
+        return None
+
+    def forward(self, ctx, h, cache, given=None):
+        x = given if given is not None else self._input(ctx, h)
         if getattr(self.mixer, "can_overwrite", False):
             y = ctx.scratch("sublayer_out", tuple(h.shape), torch.float32)
             self.mixer.forward(ctx, x, y, cache, accumulate=False)
         else:
             y = self._cleared(ctx, h)
             self.mixer.forward(ctx, x, y, cache)
-        self.mixer_norm.add_normed(ctx, h, y)
         if self.feed_forward is None:
-            return
-        x = self._input(ctx, h)
+            return self._add_normed(ctx, self.mixer_norm, h, y, "stream_rounded_next")
+        x = self._add_normed(ctx, self.mixer_norm, h, y, "stream_rounded_mid")
+        if x is None:
+            x = self._input(ctx, h)
         if getattr(self.feed_forward, "applies_output_norm", False) and getattr(self.ff_norm, "rms_parameters", None) is not None:
+            if ctx.dtype == torch.bfloat16 and getattr(self.feed_forward, "rounds_stream", False):
+                rounded = ctx.scratch("stream_rounded_next", tuple(h.shape), torch.bfloat16)
+                self.feed_forward.forward(ctx, x, h, output_norm=self.ff_norm, rounded=rounded)
+                return rounded
             self.feed_forward.forward(ctx, x, h, output_norm=self.ff_norm)
-            return
+            return None
         y = self._cleared(ctx, h)
         self.feed_forward.forward(ctx, x, y)
-        self.ff_norm.add_normed(ctx, h, y)
+        return self._add_normed(ctx, self.ff_norm, h, y, "stream_rounded_next")
 
 
 register("block", "outnorm", OutputNormBlock)

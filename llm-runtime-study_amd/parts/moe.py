@@ -26,6 +26,7 @@ class RoutedExperts(Part):
     graph_safe = True
     plan_safe = True
     applies_output_norm = True    # forward(..., output_norm=norm): residual += norm(out) instead of residual += out
+    rounds_stream = True          # forward(..., rounded=buffer): the updated stream is left there in bfloat16 as well
 
     def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int, top: int, router_bias: bool = False,
                  activation: str = "relu_squared"):
@@ -69,7 +70,7 @@ class RoutedExperts(Part):
     def flops(self, tokens, pairs):
         return 2.0 * tokens * (self.num_experts * self.hidden_size + 2 * self.top * self.hidden_size * self.intermediate_size)
 
-    def forward(self, ctx, x, residual, then_norm=None, output_norm=None):
+    def forward(self, ctx, x, residual, then_norm=None, output_norm=None, rounded=None):
         t = rows_of(x)
         x = materialize(ctx, x)
         experts, top = self.num_experts, self.top
@@ -89,10 +90,10 @@ class RoutedExperts(Part):
         outputs = ctx.scratch("moe_outputs", (rows, self.hidden_size), torch.float32)
         ops.moe_experts(outputs, hidden, self.down, sorted_pairs, tile_expert, tile, top, gather=False, relu_squared=False)
         if output_norm is None:
-            ops.moe_combine(residual, outputs, place, weights, None)
+            ops.moe_combine(residual[:t], outputs, place, weights, None, rounded=rounded)
         else:
             weight, eps = output_norm.rms_parameters()
-            ops.moe_combine(residual, outputs, place, weights, weight, eps)
+            ops.moe_combine(residual[:t], outputs, place, weights, weight, eps, rounded=rounded)
         return None
 
 

@@ -39,9 +39,12 @@ class RMSNorm(Part):
         if self.unit_offset:
             self.weight = (1.0 + self.weight.float()).contiguous()
 
-    def add_normed(self, ctx, residual, y):
-        """residual += this norm of the float32 rows y (what a sublayer gave out)."""
-        ops.norm_add(residual, y, self.weight, self.eps)
+    rounds_stream = True   # add_normed(..., rounded=buffer) also leaves the updated rows in bfloat16
+
+    def add_normed(self, ctx, residual, y, rounded=None):
+        """residual += this norm of the float32 rows y (what a sublayer gave out); rounded: a bfloat16 buffer that
+        receives the updated rows as well, for the sublayer that reads the stream next."""
+        ops.norm_add(residual, y, self.weight, self.eps, rounded)
 
     def rms_parameters(self):
         """(weight, eps): says that this norm is w * x * rsqrt(mean(x^2) + eps), so that the matrix
