@@ -37,7 +37,7 @@ ROUTED = model(211, 64, 1e-5, [
 # every expert runs for every token (no choice to differ in), a layer without feed-forward, whole heads rotated, one without
 # rotation and one without window, a convolution of one tap, more experts than a wave has lanes
 DENSE = model(157, 96, 3e-6, [
-    attention(2, 2, 64, 0.11, window=40, rot=(250000.0, 64), mlp=experts(32, 3, 3)),
+    attention(2, 2, 64, 0.11, window=40, rot=(200000.0, 64), mlp=experts(32, 3, 3)),
     delta(3, 3, 20, 28, 3, None),
     attention(4, 1, 32, 0.2, window=None, rot=None, mlp=experts(24, 70, 70)),
     delta(2, 2, 64, 64, 1, experts(64, 2, 2)),
@@ -48,6 +48,12 @@ CORES = model(300, 128, 1e-6, [
     attention(4, 2, 128, 0.09, window=100, rot=(1e6, 128), mlp=experts(64, 8, 8)),
     delta(2, 1, 128, 128, 4, experts(128, 4, 4)),
     attention(8, 4, 64, 0.125, window=33, rot=(1e4, 32), mlp=experts(64, 8, 8)),
+])
+# wide enough that prompts go through the products for many rows (the vendor library's, the grouped product with large tiles)
+WIDE = model(1000, 512, 1e-6, [
+    delta(8, 4, 64, 64, 4, experts(256, 8, 2)),
+    attention(8, 2, 64, 0.12, window=150, rot=(1e5, 32), mlp=experts(256, 4, 4)),
+    delta(4, 4, 128, 128, 2, None),
 ])
 
 

@@ -104,7 +104,7 @@ def moe_weights(width, ff, count, seed):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("width,ff,count,top,tokens", [(64, 48, 6, 2, 50), (128, 64, 70, 3, 200), (128, 128, 8, 8, 33), (40, 24, 5, 1, 7), (192, 64, 16, 4, 1),
+@pytest.mark.parametrize("width,ff,count,top,tokens", [(64, 48, 6, 2, 50), (128, 64, 70, 3, 200), (128, 128, 8, 8, 33), (40, 24, 5, 1, 7), (320, 64, 16, 4, 1),
                                                        (128, 192, 3, 2, 400), (72, 40, 2, 2, 260), (256, 320, 4, 2, 600), (512, 96, 2, 1, 700)])
 def test_grouped_expert_products_with_given_choices(dtype, width, ff, count, top, tokens):
     """The sort by expert, the two grouped products and the weighted sum, with the choices given (no routing decision to
@@ -277,6 +277,24 @@ def test_cuts_change_no_bit_in_float32(models, tmp_path):
     for key in ga:
         for position in ga[key]:
             assert torch.equal(ga[key][position], gb[key][position]), f"{key}@{position}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_wider_model_through_the_products_for_many_rows(tmp_path, dtype):
+    """Width 512 and prompts of 330 and 140 tokens: the projections of a prompt are products of hundreds of rows (the
+    vendor library's in bfloat16), the experts get dozens to hundreds of rows each (large tiles), heads of 64 and 128."""
+    raw = configs.WIDE
+    folder = configs.write_folder(raw, 21, tmp_path / "wide")
+    _, weights = plain.load_model_dir(folder)
+    rng = np.random.default_rng(4)
+    requests = {"long": rng.integers(0, raw["vocab"], 330).tolist(), "short": rng.integers(0, raw["vocab"], 140).tolist()}
+    want = {key: plain.forward(weights, raw, tokens) for key, tokens in requests.items()}
+    steps = [{"step": 0, "entries": [{"id": key, "tokens": tokens[:-6], "want": list(range(0, len(tokens) - 6, 7))} for key, tokens in requests.items()], "end": []}]
+    for i in range(6, 0, -1):
+        steps.append({"step": len(steps), "entries": [{"id": key, "tokens": [tokens[-i]], "want": [0]} for key, tokens in requests.items()],
+                      "end": list(requests) if i == 1 else []})
+    got = traces.collect(steps, run_replay(folder, dtype, steps, 512, tmp_path / "o"), raw["vocab"])
+    assert check(got, want, dtype, "routed") > 70
 
 
 # ------------------------------------------------------------------------------------- planted inputs
