@@ -32,14 +32,16 @@ __device__ __forceinline__ float silu_f(float x) { return x / (1.f + expf(-x)); 
 template <typename TP>
 __global__ void delta_prepare_kernel(const TP* __restrict__ proj, int ld, const int* __restrict__ token_request,
                                      const int* __restrict__ cu, const int* __restrict__ slot_ids,
-                                     const float* __restrict__ state, int64_t state_stride, int64_t conv_offset,
+                                     float* __restrict__ state, int64_t state_stride, int64_t conv_offset,
                                      const float* __restrict__ conv_w, int taps, int G, int H, int d, int dv,
                                      const float* __restrict__ a_log, const float* __restrict__ dt_bias,
-                                     float* __restrict__ qkv, float* __restrict__ gates) {
+                                     float* __restrict__ qkv, float* __restrict__ gates, int keep_inside) {
+  // keep_inside: every request brings one token, so this wave alone reads and writes its channels' kept inputs of its
+  // request: it moves them on itself (no delta_conv_keep launch)
   const int t = blockIdx.x, unit = blockIdx.y, lane = threadIdx.x;
   const int channels = 2 * G * d + H * dv;
   const int r = token_request[t], start = cu[r], at = t - start;
-  const float* kept = state + (int64_t)slot_ids[r] * state_stride + conv_offset;
+  float* kept = state + (int64_t)slot_ids[r] * state_stride + conv_offset;
   const bool is_v = unit >= 2 * G;
   const int c0 = is_v ? 2 * G * d + (unit - 2 * G) * dv : unit * d, n = is_v ? dv : d;
   float* out = qkv + (int64_t)t * channels + c0;
@@ -51,6 +53,7 @@ __global__ void delta_prepare_kernel(const TP* __restrict__ proj, int ld, const 
       const int s = at - (taps - 1 - j);
       const float x = s >= 0 ? to_float(proj[(int64_t)(start + s) * ld + c]) : kept[(int64_t)(taps - 1 + s) * channels + c];
       acc = fmaf(conv_w[(int64_t)c * taps + j], x, acc);
+      if (keep_inside && j > 0) kept[(int64_t)(j - 1) * channels + c] = x;      // input j of this token's window is entry j - 1 of the next one's
     }
     const float y = silu_f(acc);
     out[i] = y;
@@ -318,8 +321,9 @@ LRS_API int lrs_delta_rule(void* out, int out_dtype, const void* proj, int proj_
 #define ALL(TP, TO)                                                                                                           \
   do {                                                                                                                        \
     delta_prepare_kernel<TP><<<pgrid, WAVE, 0, s>>>((const TP*)proj, ld, token_request, cu, slot_ids, state, state_stride,    \
-                                                    conv_offset, conv_w, taps, G, H, d, dv, a_log, dt_bias, qkv, gates);      \
-    if (taps > 1)                                                                                                             \
+                                                    conv_offset, conv_w, taps, G, H, d, dv, a_log, dt_bias, qkv, gates,       \
+                                                    tokens == requests);                                                      \
+    if (taps > 1 && tokens != requests)                                                                                       \
       delta_conv_keep_kernel<TP><<<kgrid, 256, 0, s>>>((const TP*)proj, ld, cu, slot_ids, state, state_stride, conv_offset,  \
                                                        taps, channels);                                                       \
     if (tokens == requests) {        /* one token each: token r is request r's */                                             \

@@ -21,11 +21,9 @@ namespace {
 
 constexpr int ROUTE_MAX_PER_LANE = 8;     // experts up to 64 * 8
 
-__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int ld, const float* __restrict__ bias,
-                                                        int* __restrict__ ids, float* __restrict__ weights, int tokens,
-                                                        int experts, int top) {
-  const int t = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-  if (t >= tokens) return;
+// One token by one wave.
+__device__ __forceinline__ void route_token(const float* __restrict__ logits, int ld, const float* __restrict__ bias,
+                                            int* ids, float* __restrict__ weights, int t, int experts, int top, int lane) {
   float v[ROUTE_MAX_PER_LANE];
 #pragma unroll
   for (int c = 0; c < ROUTE_MAX_PER_LANE; ++c) {
@@ -71,13 +69,19 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     for (int k = WAVE; k < top; ++k) weights[(int64_t)t * top + k] /= total;
 }
 
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int ld, const float* __restrict__ bias,
+                                                        int* __restrict__ ids, float* __restrict__ weights, int tokens,
+                                                        int experts, int top) {
+  const int t = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+  if (t < tokens) route_token(logits, ld, bias, ids, weights, t, experts, top, threadIdx.x % WAVE);
+}
+
 // sorted [capacity]: the pair (token * top + choice) at each row of the sorted order, -1 for the rows that pad an
 // expert's run to whole tiles; place [pairs]: the row of each pair; tile_expert [max_tiles]: the expert of each
 // tile of `tile` rows, -1 for tiles not in use.
-__global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__ ids, int pairs, int experts, int tile,
-                                                         int* __restrict__ sorted, int capacity, int* __restrict__ place,
-                                                         int* __restrict__ tile_expert, int max_tiles) {
-  extern __shared__ int shared[];
+__device__ __forceinline__ void align_pairs(const int* ids, int pairs, int experts, int tile, int* __restrict__ sorted,
+                                            int capacity, int* __restrict__ place, int* __restrict__ tile_expert, int max_tiles,
+                                            int* shared) {
   int* count = shared;                  // [experts]
   int* first = count + experts;         // [experts + 1]: first row of each expert's run
   int* cursor = first + experts + 1;    // [experts]
@@ -104,6 +108,24 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__
     sorted[row] = i;
     place[i] = row;
   }
+}
+
+__global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__ ids, int pairs, int experts, int tile,
+                                                         int* __restrict__ sorted, int capacity, int* __restrict__ place,
+                                                         int* __restrict__ tile_expert, int max_tiles) {
+  extern __shared__ int shared[];
+  align_pairs(ids, pairs, experts, tile, sorted, capacity, place, tile_expert, max_tiles, shared);
+}
+
+// Both in one workgroup, for steps of few tokens (single tokens above all), where a launch costs more than either does.
+__global__ __launch_bounds__(1024) void moe_route_align_kernel(const float* __restrict__ logits, int ld, const float* __restrict__ bias,
+                                                               int* ids, float* __restrict__ weights, int tokens, int experts,
+                                                               int top, int tile, int* __restrict__ sorted, int capacity,
+                                                               int* __restrict__ place, int* __restrict__ tile_expert, int max_tiles) {
+  extern __shared__ int shared[];
+  for (int t = threadIdx.x / WAVE; t < tokens; t += blockDim.x / WAVE) route_token(logits, ld, bias, ids, weights, t, experts, top, threadIdx.x % WAVE);
+  __syncthreads();          // the choices are in memory for every thread of the workgroup
+  align_pairs(ids, tokens * top, experts, tile, sorted, capacity, place, tile_expert, max_tiles, shared);
 }
 
 enum { ACT_NONE = 0, ACT_RELU_SQUARED = 1 };
@@ -519,6 +541,19 @@ LRS_API int lrs_moe_align(const int* ids, int pairs, int experts, int* sorted, i
   LRS_REQUIRE(lds <= 48 * 1024, "moe_align: %d experts are too many", experts);
   moe_align_kernel<<<1, 1024, lds, (hipStream_t)stream>>>(ids, pairs, experts, tile, sorted, capacity, place, tile_expert, max_tiles);
   return lrs_check_launch("moe_align");
+}
+
+LRS_API int lrs_moe_route_align(const float* logits, int ld, const float* bias, int* ids, float* weights, int tokens, int experts,
+                                int top, int* sorted, int capacity, int* place, int* tile_expert, int max_tiles, void* stream) {
+  LRS_REQUIRE(tokens > 0 && tokens <= 256 && experts > 0 && top > 0 && top <= experts, "moe_route_align: bad sizes tokens=%d experts=%d top=%d", tokens, experts, top);
+  LRS_REQUIRE(experts <= WAVE * ROUTE_MAX_PER_LANE && ld >= experts, "moe_route_align: at most %d experts in rows of at least as many logits", WAVE * ROUTE_MAX_PER_LANE);
+  const int pairs = tokens * top, tile = lrs_moe_tile_rows(pairs, experts);
+  LRS_REQUIRE(max_tiles >= lrs_moe_max_tiles(pairs, experts), "moe_route_align: %d tiles may not hold %d pairs of %d experts", max_tiles, pairs, experts);
+  LRS_REQUIRE(capacity >= max_tiles * tile, "moe_route_align: the sorted list holds %d rows, %d tiles need %d", capacity, max_tiles, max_tiles * tile);
+  const size_t lds = (size_t)(3 * experts + 1) * sizeof(int);
+  moe_route_align_kernel<<<1, 1024, lds, (hipStream_t)stream>>>(logits, ld, bias, ids, weights, tokens, experts, top, tile, sorted, capacity, place,
+                                                                tile_expert, max_tiles);
+  return lrs_check_launch("moe_route_align");
 }
 
 // out [max_tiles * tile, n] = rows of `a` (row pair / top of the sorted list if `gather`, else the sorted row

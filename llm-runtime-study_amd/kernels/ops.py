@@ -152,6 +152,7 @@ _SIGNATURES = {
     "lrs_moe_tile_rows": (c_int, [c_int, c_int]),
     "lrs_moe_max_tiles": (c_int, [c_int, c_int]),
     "lrs_moe_route": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "lrs_moe_route_align": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p]),
     "lrs_moe_align": (c_int, [c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p]),
     "lrs_moe_experts": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
                                 c_int, c_int, c_void_p]),
@@ -194,7 +195,7 @@ def library():
 PLAN_OPS = ("lrs_add_into", "lrs_add_rmsnorm", "lrs_advance_decode", "lrs_advance_slots", "lrs_attention", "lrs_attention_decode",
             "lrs_attention_prefill", "lrs_choose_tokens", "lrs_choose_tokens_split", "lrs_copy_to_pinned", "lrs_delta_rule", "lrs_embed", "lrs_fill_i32",
             "lrs_filter_logits", "lrs_gather_rows", "lrs_gemm", "lrs_gemm_lines_add_rmsnorm", "lrs_gemm_mid_add_norm_begin", "lrs_gemm_mid_qk_prep", "lrs_gemm_mid_scaled",
-            "lrs_gemm_norm_chain", "lrs_library_gemm", "lrs_moe_align", "lrs_moe_combine", "lrs_moe_experts", "lrs_moe_route", "lrs_norm_add",
+            "lrs_gemm_norm_chain", "lrs_library_gemm", "lrs_moe_align", "lrs_moe_combine", "lrs_moe_experts", "lrs_moe_route", "lrs_moe_route_align", "lrs_norm_add",
             "lrs_qk_prep", "lrs_rmsnorm", "lrs_rope_table", "lrs_round_rows", "lrs_scale_rows", "lrs_silu_mul")
 _PLAN_INDEX = {name: index for index, name in enumerate(PLAN_OPS)}
 
@@ -1205,6 +1206,28 @@ def moe_align(ids: torch.Tensor, experts: int, sorted_pairs: torch.Tensor, place
     _need(tiles >= moe_max_tiles(pairs, experts) and sorted_pairs.numel() >= tiles * tile and place.numel() >= pairs,
           "moe_align: the lists are too short for the step")
     _launch("lrs_moe_align", _dev(ids, "ids"), pairs, experts, _dev(sorted_pairs, "sorted_pairs"), sorted_pairs.numel(), _dev(place, "place"),
+            _dev(tile_expert, "tile_expert"), tiles, _stream())
+
+
+ROUTE_ALIGN_TOKENS = 32      # steps up to which one workgroup both chooses and sorts (its 16 waves take a token each, in turns)
+
+
+def moe_route_align(logits: torch.Tensor, bias: torch.Tensor | None, ids: torch.Tensor, weights: torch.Tensor, sorted_pairs: torch.Tensor,
+                    place: torch.Tensor, tile_expert: torch.Tensor) -> None:
+    """moe_route() and moe_align() as one launch, for steps of at most ROUTE_ALIGN_TOKENS tokens."""
+    tokens, top = ids.shape
+    experts, pairs, tiles = logits.shape[1], ids.numel(), tile_expert.numel()
+    _need(tokens <= ROUTE_ALIGN_TOKENS, f"moe_route_align: at most {ROUTE_ALIGN_TOKENS} tokens")
+    _need(logits.dtype == torch.float32 and logits.shape[0] >= tokens and logits.stride(1) == 1, "moe_route_align: logits must be float32 [T, E]")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == experts and bias.is_contiguous()), "moe_route_align: bias must hold E float32 values")
+    _need(ids.dtype == torch.int32 and ids.is_contiguous() and weights.dtype == torch.float32 and weights.is_contiguous()
+          and weights.shape == ids.shape, "moe_route_align: ids must be int32 [T, top] and weights float32 [T, top]")
+    for name, t in (("sorted_pairs", sorted_pairs), ("place", place), ("tile_expert", tile_expert)):
+        _need(t.dtype == torch.int32 and t.is_contiguous(), f"moe_route_align: {name} must be contiguous int32")
+    _need(tiles >= moe_max_tiles(pairs, experts) and sorted_pairs.numel() >= tiles * moe_tile_rows(pairs, experts) and place.numel() >= pairs,
+          "moe_route_align: the lists are too short for the step")
+    _launch("lrs_moe_route_align", _dev(logits, "logits"), logits.stride(0), None if bias is None else _dev(bias, "bias"), _dev(ids, "ids"),
+            _dev(weights, "weights"), tokens, experts, top, _dev(sorted_pairs, "sorted_pairs"), sorted_pairs.numel(), _dev(place, "place"),
             _dev(tile_expert, "tile_expert"), tiles, _stream())
 
 

@@ -78,13 +78,16 @@ class RoutedExperts(Part):
         ops.gemm(logits, x, self.router, choice=kernels_of(ctx), workspace=workspace_of(ctx) if ctx.dtype == torch.bfloat16 else None)
         ids = ctx.scratch("moe_ids", (t, top), torch.int32)
         weights = ctx.scratch("moe_weights", (t, top), torch.float32)
-        ops.moe_route(logits[:, :experts], self.bias, ids, weights)
         tile, tiles = ops.moe_tile_rows(t * top, experts), ops.moe_max_tiles(t * top, experts)
         rows = tiles * tile
         sorted_pairs = ctx.scratch("moe_sorted", (rows,), torch.int32)
         place = ctx.scratch("moe_place", (t * top,), torch.int32)
         tile_expert = ctx.scratch("moe_tile_expert", (tiles,), torch.int32)
-        ops.moe_align(ids, experts, sorted_pairs, place, tile_expert)
+        if t <= ops.ROUTE_ALIGN_TOKENS:        # few tokens: the choice and the sort in one launch
+            ops.moe_route_align(logits[:, :experts], self.bias, ids, weights, sorted_pairs, place, tile_expert)
+        else:
+            ops.moe_route(logits[:, :experts], self.bias, ids, weights)
+            ops.moe_align(ids, experts, sorted_pairs, place, tile_expert)
         hidden = ctx.scratch("moe_hidden", (rows, self.intermediate_size), ctx.dtype)
         ops.moe_experts(hidden, x, self.up, sorted_pairs, tile_expert, tile, top, gather=True, relu_squared=True)
         outputs = ctx.scratch("moe_outputs", (rows, self.hidden_size), torch.float32)
