@@ -2,8 +2,8 @@
 fixed-size per-request state.
 
 What each schedule entry of the model keeps between steps is declared by its mixer:
-  PagedKVNeed(nkv, d, window, dtype)  keys and values of every position, or of a sliding window, kept in `dtype`
-                               (None: the run's activation dtype);
+  PagedKVNeed(nkv, d, window, dtype, values)  keys and values of every position, or of a sliding window, kept in `dtype`
+                               (None: the run's activation dtype); values False: key pages alone (one row a position);
   StateNeed(shape, dtype)      a state of fixed size;
   ("from", j)                  nothing of its own: it reads the cache of entry j;
   None                         nothing.
@@ -154,9 +154,10 @@ class CacheManager:
                 v_shape = (num_pages + 1, group.need.num_kv_heads, group.need.head_dim, page_size)
                 for position in group.entries:
                     group.k[position] = torch.zeros(k_shape, dtype=group.dtype, device=self.device)
-                    group.v[position] = torch.zeros(v_shape, dtype=group.dtype, device=self.device)
                     self.layer_caches[position].k_pages = group.k[position]
-                    self.layer_caches[position].v_pages = group.v[position]
+                    if group.need.values:
+                        group.v[position] = torch.zeros(v_shape, dtype=group.dtype, device=self.device)
+                        self.layer_caches[position].v_pages = group.v[position]
 
     # ------------------------------------------------------------------ sizes
     @property
@@ -183,7 +184,7 @@ class CacheManager:
         return max((g.pool.used_pages for g in self.groups), default=0) * self.page_size
 
     def bytes_per_token(self) -> int:
-        return sum(2 * len(g.entries) * g.need.num_kv_heads * g.need.head_dim * torch.empty(0, dtype=g.dtype).element_size()
+        return sum((2 if g.need.values else 1) * len(g.entries) * g.need.num_kv_heads * g.need.head_dim * torch.empty(0, dtype=g.dtype).element_size()
                    for g in self.groups)
 
     def trash_page(self, group: int = 0) -> int:

@@ -72,7 +72,9 @@ def _load_builtin() -> None:
     _builtin_loaded = True
     from ..models.qwen3 import build_spec
     from ..text.chat import format_qwen3_chat
+    from ..models.napizen import build_spec as build_napizen
     from ..models.nobodra import build_spec as build_nobodra
+    from .napizen import NapizenConfig
     from .nobodra import NobodraConfig
     from .qwen3 import Qwen3Config
 
@@ -80,6 +82,8 @@ def _load_builtin() -> None:
         register_architecture(Qwen3Config.ARCHITECTURE, Qwen3Config, build_spec, chat_template=format_qwen3_chat)
     if NobodraConfig.ARCHITECTURE not in _ARCHITECTURES:
         register_architecture(NobodraConfig.ARCHITECTURE, NobodraConfig, build_nobodra)      # token ids only: it has no chat template
+    if NapizenConfig.ARCHITECTURE not in _ARCHITECTURES:
+        register_architecture(NapizenConfig.ARCHITECTURE, NapizenConfig, build_napizen)      # token ids only as well
     import importlib
     import os
 

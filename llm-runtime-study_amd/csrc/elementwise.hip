@@ -226,19 +226,20 @@ LRS_API int lrs_add_rmsnorm(void* out, int out_dtype, float* x, const void* y, c
 // cos/sin [tokens, half] of angle = float(position) * inv_freq[i], all in float32.
 __global__ void rope_table_kernel(float* __restrict__ cosv, float* __restrict__ sinv,
                                   const int* __restrict__ positions,
-                                  const float* __restrict__ inv_freq, int half) {
+                                  const float* __restrict__ inv_freq, int half, float magnitude) {
+  // magnitude: both tables times this (1 for a plain rotation; frequency scalings that stretch long contexts come with one)
   const float p = (float)positions[blockIdx.x];
   for (int i = threadIdx.x; i < half; i += blockDim.x) {
     const float angle = p * inv_freq[i];
-    cosv[(int64_t)blockIdx.x * half + i] = cosf(angle);
-    sinv[(int64_t)blockIdx.x * half + i] = sinf(angle);
+    cosv[(int64_t)blockIdx.x * half + i] = magnitude == 1.0f ? cosf(angle) : cosf(angle) * magnitude;
+    sinv[(int64_t)blockIdx.x * half + i] = magnitude == 1.0f ? sinf(angle) : sinf(angle) * magnitude;
   }
 }
 
 LRS_API int lrs_rope_table(float* cosv, float* sinv, const int* positions, const float* inv_freq,
-                           int tokens, int half, void* stream) {
+                           int tokens, int half, float magnitude, void* stream) {
   LRS_REQUIRE(tokens > 0 && half > 0, "rope_table: tokens=%d half=%d must be positive", tokens, half);
-  rope_table_kernel<<<dim3(tokens), dim3(64), 0, (hipStream_t)stream>>>(cosv, sinv, positions, inv_freq, half);
+  rope_table_kernel<<<dim3(tokens), dim3(64), 0, (hipStream_t)stream>>>(cosv, sinv, positions, inv_freq, half, magnitude);
   return lrs_check_launch("rope_table");
 }
 
@@ -857,4 +858,92 @@ LRS_API int lrs_round_rows(void* out, int out_dtype, const float* x, int64_t n, 
   else if (out_dtype == LRS_F32) round_rows_kernel<float><<<blocks, 256, 0, (hipStream_t)stream>>>((float*)out, x, n);
   else return lrs_fail("round_rows: unknown dtype %d", out_dtype);
   return lrs_check_launch("round_rows");
+}
+
+// ------------------------------------------------ layer norm (mean taken off, a weight, no bias)
+// out = w * (x - mean) / sqrt(variance + eps), the variance being the mean of the squared deviations; x is a float32
+// row (optionally picked through `rows`), statistics float32, the result rounded once to the output dtype.
+template <typename TW, typename TO>
+__global__ __launch_bounds__(1024) void layernorm_kernel(TO* __restrict__ out, const float* __restrict__ x, const TW* __restrict__ weight,
+                                                        const int* __restrict__ rows, int hidden, float eps) {
+  __shared__ float scratch[16];
+  const int64_t src_row = rows ? rows[blockIdx.x] : blockIdx.x;
+  const float* src = x + src_row * hidden;
+  TO* dst = out + (int64_t)blockIdx.x * hidden;
+  float sum = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) sum += src[i];
+  const float mean = block_sum(sum, scratch) / (float)hidden;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float d = src[i] - mean;
+    ss = fmaf(d, d, ss);
+  }
+  const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)hidden + eps);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = from_float<TO>((src[i] - mean) * inv * to_float(weight[i]));
+}
+LRS_API int lrs_layernorm(void* out, int out_dtype, const float* x, const void* weight, int w_dtype, const int* rows, int n_rows, int hidden,
+                          float eps, void* stream) {
+  LRS_REQUIRE(n_rows > 0 && hidden > 0 && eps > 0.f, "layernorm: bad sizes rows=%d hidden=%d", n_rows, hidden);
+  const int threads = hidden >= 2048 ? 1024 : 256;
+  hipStream_t s = (hipStream_t)stream;
+#define LRS_LN(TW, TO) layernorm_kernel<TW, TO><<<n_rows, threads, 0, s>>>((TO*)out, x, (const TW*)weight, rows, hidden, eps)
+  if (w_dtype == LRS_F32 && out_dtype == LRS_F32) LRS_LN(float, float);
+  else if (w_dtype == LRS_F32 && out_dtype == LRS_BF16) LRS_LN(float, bf16);
+  else if (w_dtype == LRS_BF16 && out_dtype == LRS_F32) LRS_LN(bf16, float);
+  else if (w_dtype == LRS_BF16 && out_dtype == LRS_BF16) LRS_LN(bf16, bf16);
+  else return lrs_fail("layernorm: unknown dtypes %d %d", w_dtype, out_dtype);
+#undef LRS_LN
+  return lrs_check_launch("layernorm");
+}
+
+// The layer arrangement that normalises the sum: residual[r] = layer norm of (alpha * residual[r] + y[r]), all float32,
+// in place.  The sum is written where the row was and read again by the thread that wrote it.  With `rounded` the new
+// row is also left in bfloat16, for the sublayer that reads the stream next.
+template <typename TW>
+__global__ __launch_bounds__(1024) void scale_add_layernorm_kernel(float* __restrict__ residual, const float* __restrict__ y, float alpha,
+                                                                  const TW* __restrict__ weight, int hidden, float eps,
+                                                                  bf16* __restrict__ rounded) {
+  __shared__ float scratch[16];
+  const float* src = y + (int64_t)blockIdx.x * hidden;
+  float* dst = residual + (int64_t)blockIdx.x * hidden;
+  float sum = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float v = fmaf(alpha, dst[i], src[i]);
+    dst[i] = v;
+    sum += v;
+  }
+  const float mean = block_sum(sum, scratch) / (float)hidden;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float d = dst[i] - mean;
+    ss = fmaf(d, d, ss);
+  }
+  const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)hidden + eps);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float v = (dst[i] - mean) * inv * to_float(weight[i]);
+    dst[i] = v;
+    if (rounded) rounded[(int64_t)blockIdx.x * hidden + i] = (bf16)v;
+  }
+}
+LRS_API int lrs_scale_add_layernorm(float* residual, const float* y, float alpha, const void* weight, int w_dtype, int n_rows, int hidden,
+                                    float eps, void* rounded, void* stream) {
+  LRS_REQUIRE(n_rows > 0 && hidden > 0 && eps > 0.f, "scale_add_layernorm: bad sizes rows=%d hidden=%d", n_rows, hidden);
+  const int threads = hidden >= 2048 ? 1024 : 256;
+  hipStream_t s = (hipStream_t)stream;
+  if (w_dtype == LRS_F32) scale_add_layernorm_kernel<float><<<n_rows, threads, 0, s>>>(residual, y, alpha, (const float*)weight, hidden, eps, (bf16*)rounded);
+  else if (w_dtype == LRS_BF16) scale_add_layernorm_kernel<bf16><<<n_rows, threads, 0, s>>>(residual, y, alpha, (const bf16*)weight, hidden, eps, (bf16*)rounded);
+  else return lrs_fail("scale_add_layernorm: unknown weight dtype %d", w_dtype);
+  return lrs_check_launch("scale_add_layernorm");
+}
+
+// ------------------------------------------------ soft cap
+// x = cap * tanh(x / cap), in place on float32 values (logits).
+__global__ void soft_cap_kernel(float* __restrict__ x, int64_t n, float cap) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) x[i] = cap * tanhf(x[i] / cap);
+}
+LRS_API int lrs_soft_cap(float* x, int64_t n, float cap, void* stream) {
+  LRS_REQUIRE(n > 0 && cap > 0.f, "soft_cap: nothing to do, or a cap that is not positive");
+  const int blocks = (int)((n + 1023) / 1024 < 4096 ? (n + 1023) / 1024 : 4096);
+  soft_cap_kernel<<<blocks, 256, 0, (hipStream_t)stream>>>(x, n, cap);
+  return lrs_check_launch("soft_cap");
 }

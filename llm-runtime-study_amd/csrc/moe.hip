@@ -69,11 +69,116 @@ __device__ __forceinline__ void route_token(const float* __restrict__ logits, in
     for (int k = WAVE; k < top; ++k) weights[(int64_t)t * top + k] /= total;
 }
 
+// How a token's experts are chosen and weighted.
+//   ROUTE_SOFTMAX_CHOSEN  the largest (logit + bias); weights: the softmax over the chosen (logit + bias) alone
+//   ROUTE_SIGMOID         scores s = sigmoid(logit); the largest (s + bias) are chosen, the bias taking part in the
+//                         choice only; weights: the chosen s divided by their sum (+ 1e-20), times `scale`.  With
+//                         groups > 0 the experts form that many equal groups of neighbours, a group's score is the sum of
+//                         its two largest (s + bias), and only experts of the `keep` best groups can be chosen.
+enum { ROUTE_SOFTMAX_CHOSEN = 0, ROUTE_SIGMOID = 1 };
+struct RouteRule {
+  int kind, groups, keep;
+  float scale;
+};
+
+// The lowest index among the lanes' elements that equal `best` (1 << 30 if none).
+__device__ __forceinline__ int route_where(const float (&v)[ROUTE_MAX_PER_LANE], float best, int lane) {
+  int where = 1 << 30;
+#pragma unroll
+  for (int c = ROUTE_MAX_PER_LANE - 1; c >= 0; --c)
+    if (v[c] == best) where = lane + WAVE * c;
+#pragma unroll
+  for (int off = WAVE / 2; off > 0; off >>= 1) where = min(where, __shfl_xor(where, off, WAVE));
+  return where;
+}
+__device__ __forceinline__ float route_max(const float (&v)[ROUTE_MAX_PER_LANE]) {
+  float best = -INFINITY;
+#pragma unroll
+  for (int c = 0; c < ROUTE_MAX_PER_LANE; ++c) best = fmaxf(best, v[c]);
+  return wave_max(best);
+}
+
+// One token by one wave, ROUTE_SIGMOID.
+__device__ __forceinline__ void route_token_sigmoid(const float* __restrict__ logits, int ld, const float* __restrict__ bias,
+                                                    int* ids, float* __restrict__ weights, int t, int experts, int top, int lane,
+                                                    const RouteRule rule) {
+  float s[ROUTE_MAX_PER_LANE], v[ROUTE_MAX_PER_LANE];
+#pragma unroll
+  for (int c = 0; c < ROUTE_MAX_PER_LANE; ++c) {
+    const int e = lane + WAVE * c;
+    s[c] = e < experts ? 1.0f / (1.0f + expf(-logits[(int64_t)t * ld + e])) : 0.f;
+    v[c] = e < experts ? s[c] + (bias ? bias[e] : 0.f) : -INFINITY;
+  }
+  if (rule.groups > 0 && rule.keep < rule.groups) {
+    const int per = experts / rule.groups;
+    float score[ROUTE_MAX_PER_LANE];       // of group lane + WAVE * c
+#pragma unroll
+    for (int c = 0; c < ROUTE_MAX_PER_LANE; ++c) score[c] = -INFINITY;
+    for (int g = 0; g < rule.groups; ++g) {
+      float mine[ROUTE_MAX_PER_LANE];
+#pragma unroll
+      for (int c = 0; c < ROUTE_MAX_PER_LANE; ++c) mine[c] = (lane + WAVE * c) / per == g ? v[c] : -INFINITY;
+      const float first = route_max(mine);
+      float sum = first;
+      if (per > 1) {
+        const int where = route_where(mine, first, lane);
+#pragma unroll
+        for (int c = 0; c < ROUTE_MAX_PER_LANE; ++c)
+          if (lane + WAVE * c == where) mine[c] = -INFINITY;
+        sum = first + route_max(mine);
+      }
+#pragma unroll
+      for (int c = 0; c < ROUTE_MAX_PER_LANE; ++c)
+        if (lane + WAVE * c == g) score[c] = sum;
+    }
+    bool kept[ROUTE_MAX_PER_LANE];
+#pragma unroll
+    for (int c = 0; c < ROUTE_MAX_PER_LANE; ++c) kept[c] = false;
+    for (int k = 0; k < rule.keep; ++k) {
+      const float best = route_max(score);
+      int where = route_where(score, best, lane);
+      if (where >= rule.groups) where = k;   // scores that are not numbers: any group
+#pragma unroll
+      for (int c = 0; c < ROUTE_MAX_PER_LANE; ++c) {
+        if (lane + WAVE * c == where) score[c] = -INFINITY;
+        if ((lane + WAVE * c) / per == where) kept[c] = true;
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < ROUTE_MAX_PER_LANE; ++c)
+      if (!kept[c]) v[c] = -INFINITY;
+  }
+  float total = 0.f;
+  for (int k = 0; k < top; ++k) {
+    const float best = route_max(v);
+    int where = route_where(v, best, lane);
+    if (where >= experts) where = k;    // scores that are not numbers: any expert, never an index outside the table
+    float own = 0.f;
+#pragma unroll
+    for (int c = 0; c < ROUTE_MAX_PER_LANE; ++c)
+      if (lane + WAVE * c == where) {
+        v[c] = -INFINITY;
+        own = s[c];
+      }
+    const float w = __shfl(own, where % WAVE, WAVE);
+    total += w;
+    if (lane == 0) {
+      ids[(int64_t)t * top + k] = where;
+      weights[(int64_t)t * top + k] = w;
+    }
+  }
+  // the same lane wrote them: it reads its own stores
+  if (lane == 0)
+    for (int k = 0; k < top; ++k) weights[(int64_t)t * top + k] = weights[(int64_t)t * top + k] / (total + 1e-20f) * rule.scale;
+}
+
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int ld, const float* __restrict__ bias,
                                                         int* __restrict__ ids, float* __restrict__ weights, int tokens,
-                                                        int experts, int top) {
+                                                        int experts, int top, const RouteRule rule) {
   const int t = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
-  if (t < tokens) route_token(logits, ld, bias, ids, weights, t, experts, top, threadIdx.x % WAVE);
+  if (t >= tokens) return;
+  if (rule.kind == ROUTE_SIGMOID) route_token_sigmoid(logits, ld, bias, ids, weights, t, experts, top, threadIdx.x % WAVE, rule);
+  else route_token(logits, ld, bias, ids, weights, t, experts, top, threadIdx.x % WAVE);
 }
 
 // sorted [capacity]: the pair (token * top + choice) at each row of the sorted order, -1 for the rows that pad an
@@ -121,9 +226,13 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__
 __global__ __launch_bounds__(1024) void moe_route_align_kernel(const float* __restrict__ logits, int ld, const float* __restrict__ bias,
                                                                int* ids, float* __restrict__ weights, int tokens, int experts,
                                                                int top, int tile, int* __restrict__ sorted, int capacity,
-                                                               int* __restrict__ place, int* __restrict__ tile_expert, int max_tiles) {
+                                                               int* __restrict__ place, int* __restrict__ tile_expert, int max_tiles,
+                                                               const RouteRule rule) {
   extern __shared__ int shared[];
-  for (int t = threadIdx.x / WAVE; t < tokens; t += blockDim.x / WAVE) route_token(logits, ld, bias, ids, weights, t, experts, top, threadIdx.x % WAVE);
+  for (int t = threadIdx.x / WAVE; t < tokens; t += blockDim.x / WAVE) {
+    if (rule.kind == ROUTE_SIGMOID) route_token_sigmoid(logits, ld, bias, ids, weights, t, experts, top, threadIdx.x % WAVE, rule);
+    else route_token(logits, ld, bias, ids, weights, t, experts, top, threadIdx.x % WAVE);
+  }
   __syncthreads();          // the choices are in memory for every thread of the workgroup
   align_pairs(ids, tokens * top, experts, tile, sorted, capacity, place, tile_expert, max_tiles, shared);
 }
@@ -522,12 +631,28 @@ LRS_API int lrs_moe_max_tiles(int pairs, int experts) {
   return pairs < padded ? pairs : padded;
 }
 
+static int check_rule(const char* who, int kind, int groups, int keep, float scale, int experts, int top) {
+  LRS_REQUIRE(kind == ROUTE_SOFTMAX_CHOSEN || kind == ROUTE_SIGMOID, "%s: unknown routing rule %d", who, kind);
+  if (kind == ROUTE_SOFTMAX_CHOSEN) {
+    LRS_REQUIRE(groups == 0, "%s: groups of experts come with the sigmoid rule only", who);
+    return 0;
+  }
+  LRS_REQUIRE(scale > 0.f, "%s: the weights' scale must be positive", who);
+  if (groups > 0) {
+    LRS_REQUIRE(experts % groups == 0 && keep > 0 && keep <= groups, "%s: %d experts do not form %d equal groups of which %d are kept", who, experts, groups, keep);
+    LRS_REQUIRE((int64_t)keep * (experts / groups) >= top, "%s: %d groups of %d experts hold fewer than the %d to choose", who, keep, experts / groups, top);
+  }
+  return 0;
+}
+
+// rule, groups, keep, scale: see RouteRule (0, 0, 0, 1 for the softmax over the chosen logits).
 LRS_API int lrs_moe_route(const float* logits, int ld, const float* bias, int* ids, float* weights, int tokens, int experts,
-                          int top, void* stream) {
+                          int top, int rule, int groups, int keep, float scale, void* stream) {
+  if (int rc = check_rule("moe_route", rule, groups, keep, scale, experts, top)) return rc;
   LRS_REQUIRE(tokens > 0 && experts > 0 && top > 0 && top <= experts, "moe_route: bad sizes tokens=%d experts=%d top=%d", tokens, experts, top);
   LRS_REQUIRE(experts <= WAVE * ROUTE_MAX_PER_LANE, "moe_route: at most %d experts, got %d", WAVE * ROUTE_MAX_PER_LANE, experts);
   LRS_REQUIRE(ld >= experts, "moe_route: rows of %d logits hold fewer than %d experts", ld, experts);
-  moe_route_kernel<<<(tokens + 3) / 4, 256, 0, (hipStream_t)stream>>>(logits, ld, bias, ids, weights, tokens, experts, top);
+  moe_route_kernel<<<(tokens + 3) / 4, 256, 0, (hipStream_t)stream>>>(logits, ld, bias, ids, weights, tokens, experts, top, RouteRule{rule, groups, keep, scale});
   return lrs_check_launch("moe_route");
 }
 
@@ -544,7 +669,9 @@ LRS_API int lrs_moe_align(const int* ids, int pairs, int experts, int* sorted, i
 }
 
 LRS_API int lrs_moe_route_align(const float* logits, int ld, const float* bias, int* ids, float* weights, int tokens, int experts,
-                                int top, int* sorted, int capacity, int* place, int* tile_expert, int max_tiles, void* stream) {
+                                int top, int* sorted, int capacity, int* place, int* tile_expert, int max_tiles, int rule, int groups, int keep,
+                                float scale, void* stream) {
+  if (int rc = check_rule("moe_route_align", rule, groups, keep, scale, experts, top)) return rc;
   LRS_REQUIRE(tokens > 0 && tokens <= 256 && experts > 0 && top > 0 && top <= experts, "moe_route_align: bad sizes tokens=%d experts=%d top=%d", tokens, experts, top);
   LRS_REQUIRE(experts <= WAVE * ROUTE_MAX_PER_LANE && ld >= experts, "moe_route_align: at most %d experts in rows of at least as many logits", WAVE * ROUTE_MAX_PER_LANE);
   const int pairs = tokens * top, tile = lrs_moe_tile_rows(pairs, experts);
@@ -552,7 +679,7 @@ LRS_API int lrs_moe_route_align(const float* logits, int ld, const float* bias, 
   LRS_REQUIRE(capacity >= max_tiles * tile, "moe_route_align: the sorted list holds %d rows, %d tiles need %d", capacity, max_tiles, max_tiles * tile);
   const size_t lds = (size_t)(3 * experts + 1) * sizeof(int);
   moe_route_align_kernel<<<1, 1024, lds, (hipStream_t)stream>>>(logits, ld, bias, ids, weights, tokens, experts, top, tile, sorted, capacity, place,
-                                                                tile_expert, max_tiles);
+                                                                tile_expert, max_tiles, RouteRule{rule, groups, keep, scale});
   return lrs_check_launch("moe_route_align");
 }
 

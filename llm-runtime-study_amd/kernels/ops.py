@@ -81,7 +81,7 @@ _SIGNATURES = {
     "lrs_embed": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_void_p]),
     "lrs_rmsnorm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_void_p]),
     "lrs_add_rmsnorm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_void_p]),
-    "lrs_rope_table": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
+    "lrs_rope_table": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p]),
     "lrs_qk_prep": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_float,
                             c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "lrs_gemm_mid_qk_prep": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_float, c_int, c_int, c_int,
@@ -151,11 +151,20 @@ _SIGNATURES = {
                                c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p]),
     "lrs_moe_tile_rows": (c_int, [c_int, c_int]),
     "lrs_moe_max_tiles": (c_int, [c_int, c_int]),
-    "lrs_moe_route": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
-    "lrs_moe_route_align": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p]),
+    "lrs_moe_route": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p]),
+    "lrs_moe_route_align": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int,
+                                    c_int, c_int, c_int, c_float, c_void_p]),
     "lrs_moe_align": (c_int, [c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p]),
     "lrs_moe_experts": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
                                 c_int, c_int, c_void_p]),
+    "lrs_layernorm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_void_p]),
+    "lrs_scale_add_layernorm": (c_int, [c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_int, c_float, c_void_p, c_void_p]),
+    "lrs_soft_cap": (c_int, [c_void_p, c_int64, c_float, c_void_p]),
+    "lrs_latent_prep": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p,
+                                c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+    "lrs_head_gemm": (c_int, [c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "lrs_latent_attention": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                     c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
     "lrs_moe_combine": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p]),
 }
 
@@ -195,8 +204,8 @@ def library():
 PLAN_OPS = ("lrs_add_into", "lrs_add_rmsnorm", "lrs_advance_decode", "lrs_advance_slots", "lrs_attention", "lrs_attention_decode",
             "lrs_attention_prefill", "lrs_choose_tokens", "lrs_choose_tokens_split", "lrs_copy_to_pinned", "lrs_delta_rule", "lrs_embed", "lrs_fill_i32",
             "lrs_filter_logits", "lrs_gather_rows", "lrs_gemm", "lrs_gemm_lines_add_rmsnorm", "lrs_gemm_mid_add_norm_begin", "lrs_gemm_mid_qk_prep", "lrs_gemm_mid_scaled",
-            "lrs_gemm_norm_chain", "lrs_library_gemm", "lrs_moe_align", "lrs_moe_combine", "lrs_moe_experts", "lrs_moe_route", "lrs_moe_route_align", "lrs_norm_add",
-            "lrs_qk_prep", "lrs_rmsnorm", "lrs_rope_table", "lrs_round_rows", "lrs_scale_rows", "lrs_silu_mul")
+            "lrs_gemm_norm_chain", "lrs_head_gemm", "lrs_latent_attention", "lrs_latent_prep", "lrs_layernorm", "lrs_library_gemm", "lrs_moe_align", "lrs_moe_combine", "lrs_moe_experts", "lrs_moe_route", "lrs_moe_route_align", "lrs_norm_add",
+            "lrs_qk_prep", "lrs_rmsnorm", "lrs_rope_table", "lrs_round_rows", "lrs_scale_add_layernorm", "lrs_scale_rows", "lrs_silu_mul", "lrs_soft_cap")
 _PLAN_INDEX = {name: index for index, name in enumerate(PLAN_OPS)}
 
 
@@ -457,13 +466,45 @@ def norm_add(residual: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps:
             _rounded(rounded, n_rows, hidden, "norm_add"), _stream())
 
 
-def rope_table(cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor) -> None:
+def layernorm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float, rows: torch.Tensor | None = None) -> None:
+    """out = weight * (x - mean) / sqrt(variance + eps) per float32 row of x (of the rows listed in `rows` if given)."""
+    n_rows, hidden = out.shape
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.shape[1] == hidden and x.is_contiguous() and out.is_contiguous(), "layernorm: x must be contiguous float32 [*, H] and out [rows, H]")
+    _need(weight.is_contiguous() and weight.numel() == hidden, f"layernorm: weight must hold {hidden} values")
+    if rows is None:
+        _need(x.shape[0] >= n_rows, "layernorm: x has fewer rows than out")
+    else:
+        _need(rows.dtype == torch.int32 and rows.numel() >= n_rows and rows.is_contiguous(), "layernorm: rows must be int32")
+    _launch("lrs_layernorm", _dev(out, "out"), dtype_code(out.dtype), _dev(x, "x"), _dev(weight, "weight"), dtype_code(weight.dtype),
+            None if rows is None else _dev(rows, "rows"), n_rows, hidden, eps, _stream())
+
+
+def scale_add_layernorm(residual: torch.Tensor, y: torch.Tensor, alpha: float, weight: torch.Tensor, eps: float,
+                        rounded: torch.Tensor | None = None) -> None:
+    """residual = layer norm (weight, eps) of alpha * residual + y, float32 rows in place; rounded: bfloat16 [T, H] that
+    receives the new rows as well."""
+    n_rows, hidden = residual.shape
+    _need(residual.dtype == torch.float32 and y.dtype == torch.float32 and y.shape == residual.shape and residual.is_contiguous() and y.is_contiguous(),
+          "scale_add_layernorm: residual and y must be contiguous float32 of one shape")
+    _need(weight.is_contiguous() and weight.numel() == hidden, f"scale_add_layernorm: weight must hold {hidden} values")
+    _launch("lrs_scale_add_layernorm", _dev(residual, "residual"), _dev(y, "y"), alpha, _dev(weight, "weight"), dtype_code(weight.dtype), n_rows,
+            hidden, eps, _rounded(rounded, n_rows, hidden, "scale_add_layernorm"), _stream())
+
+
+def soft_cap(x: torch.Tensor, cap: float) -> None:
+    """x = cap * tanh(x / cap), in place on contiguous float32 values."""
+    _need(x.dtype == torch.float32 and x.is_contiguous() and x.numel() > 0, "soft_cap: x must be contiguous float32")
+    _launch("lrs_soft_cap", _dev(x, "x"), x.numel(), cap, _stream())
+
+
+def rope_table(cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor, magnitude: float = 1.0) -> None:
+    """cos, sin [T, half] = magnitude * cos / sin of (position * inv_freq), float32."""
     tokens, half = cos.shape
     _need(cos.is_contiguous() and sin.is_contiguous() and sin.shape == cos.shape, "rope_table: cos and sin must be contiguous [T, half]")
     _need(inv_freq.numel() == half and inv_freq.is_contiguous(), "rope_table: inv_freq must hold `half` values")
     _need(positions.dtype == torch.int32 and positions.numel() >= tokens and positions.is_contiguous(), "rope_table: positions must be int32 [T]")
     _launch("lrs_rope_table", _dev(cos, "cos", torch.float32), _dev(sin, "sin", torch.float32), _dev(positions, "positions"),
-                                    _dev(inv_freq, "inv_freq", torch.float32), tokens, half, _stream())
+                                    _dev(inv_freq, "inv_freq", torch.float32), tokens, half, magnitude, _stream())
 
 
 def qk_prep(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight, k_weight, eps: float, cos, sin,
@@ -1184,8 +1225,30 @@ def moe_max_tiles(pairs: int, experts: int) -> int:
     return min(pairs, pairs // moe_tile_rows(pairs, experts) + experts)
 
 
-def moe_route(logits: torch.Tensor, bias: torch.Tensor | None, ids: torch.Tensor, weights: torch.Tensor) -> None:
-    """ids, weights [T, top]: per token the `top` largest of logits [T, E] (+ bias) and the softmax over those alone."""
+@dataclass(frozen=True)
+class RouteRule:
+    """How routed experts are chosen and weighted.  kind "softmax_chosen": the largest (logit + bias), weighted by the
+    softmax over the chosen (logit + bias) alone.  kind "sigmoid": scores s = sigmoid(logit); the largest (s + bias) are
+    chosen (the bias takes part in the choice only), weighted by the chosen s over their sum (+ 1e-20), times `scale`; with
+    `groups` the experts form that many equal groups of neighbours, a group scores the sum of its two largest (s + bias),
+    and only experts of the `keep` best groups can be chosen."""
+    kind: str = "softmax_chosen"
+    groups: int = 0
+    keep: int = 0
+    scale: float = 1.0
+
+    KINDS = ("softmax_chosen", "sigmoid")
+
+    def words(self) -> tuple:
+        _need(self.kind in self.KINDS, f"unknown routing rule {self.kind!r}; known: {', '.join(self.KINDS)}")
+        return self.KINDS.index(self.kind), self.groups, self.keep, float(self.scale)
+
+
+DEFAULT_RULE = RouteRule()
+
+
+def moe_route(logits: torch.Tensor, bias: torch.Tensor | None, ids: torch.Tensor, weights: torch.Tensor, rule: RouteRule = DEFAULT_RULE) -> None:
+    """ids, weights [T, top]: per token the `top` experts of logits [T, E] that `rule` chooses, and their weights."""
     tokens, top = ids.shape
     experts = logits.shape[1]
     _need(logits.dtype == torch.float32 and logits.shape[0] >= tokens and logits.stride(1) == 1, "moe_route: logits must be float32 [T, E]")
@@ -1193,7 +1256,7 @@ def moe_route(logits: torch.Tensor, bias: torch.Tensor | None, ids: torch.Tensor
     _need(ids.dtype == torch.int32 and ids.is_contiguous() and weights.dtype == torch.float32 and weights.is_contiguous()
           and weights.shape == ids.shape, "moe_route: ids must be int32 [T, top] and weights float32 [T, top]")
     _launch("lrs_moe_route", _dev(logits, "logits"), logits.stride(0), None if bias is None else _dev(bias, "bias"), _dev(ids, "ids"),
-            _dev(weights, "weights"), tokens, experts, top, _stream())
+            _dev(weights, "weights"), tokens, experts, top, *rule.words(), _stream())
 
 
 def moe_align(ids: torch.Tensor, experts: int, sorted_pairs: torch.Tensor, place: torch.Tensor, tile_expert: torch.Tensor) -> None:
@@ -1213,7 +1276,7 @@ ROUTE_ALIGN_TOKENS = 32      # steps up to which one workgroup both chooses and 
 
 
 def moe_route_align(logits: torch.Tensor, bias: torch.Tensor | None, ids: torch.Tensor, weights: torch.Tensor, sorted_pairs: torch.Tensor,
-                    place: torch.Tensor, tile_expert: torch.Tensor) -> None:
+                    place: torch.Tensor, tile_expert: torch.Tensor, rule: RouteRule = DEFAULT_RULE) -> None:
     """moe_route() and moe_align() as one launch, for steps of at most ROUTE_ALIGN_TOKENS tokens."""
     tokens, top = ids.shape
     experts, pairs, tiles = logits.shape[1], ids.numel(), tile_expert.numel()
@@ -1228,7 +1291,7 @@ def moe_route_align(logits: torch.Tensor, bias: torch.Tensor | None, ids: torch.
           "moe_route_align: the lists are too short for the step")
     _launch("lrs_moe_route_align", _dev(logits, "logits"), logits.stride(0), None if bias is None else _dev(bias, "bias"), _dev(ids, "ids"),
             _dev(weights, "weights"), tokens, experts, top, _dev(sorted_pairs, "sorted_pairs"), sorted_pairs.numel(), _dev(place, "place"),
-            _dev(tile_expert, "tile_expert"), tiles, _stream())
+            _dev(tile_expert, "tile_expert"), tiles, *rule.words(), _stream())
 
 
 def moe_experts(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, sorted_pairs: torch.Tensor, tile_expert: torch.Tensor, tile: int, top: int,
@@ -1263,3 +1326,57 @@ def moe_combine(residual: torch.Tensor, rows: torch.Tensor, place: torch.Tensor,
     _launch("lrs_moe_combine", _dev(residual, "residual"), _dev(rows, "rows"), tokens, hidden, _dev(place, "place"), _dev(weights, "weights"), top,
             None if norm_weight is None else _dev(norm_weight, "norm_weight"), 0 if norm_weight is None else dtype_code(norm_weight.dtype), eps,
             _rounded(rounded, tokens, hidden, "moe_combine"), _stream())
+
+
+# ------------------------------------------------------------------- latent attention
+def latent_prep(proj: torch.Tensor, q_col: int, kv_col: int, heads: int, dim: int, rot: int, rank: int, norm_weight: torch.Tensor, eps: float,
+                cos: torch.Tensor | None, sin: torch.Tensor | None, pages: torch.Tensor, slots: torch.Tensor, queries: torch.Tensor) -> None:
+    """Per token of proj [T, columns]: the RMS norm (norm_weight, eps) of the `rank` latent values at column kv_col and the
+    rotation (pairs 2i, 2i + 1; cos, sin [T, rot / 2], None: none) of the `rot` shared key values behind them, written into
+    the token's row of pages [P, 1, page, rank + rot] (slots[t] < 0: not kept); and the rotation of the last `rot` of the
+    dim + rot values of every head's query (from column q_col on) into queries [T, heads, rank + rot][..., rank:]."""
+    tokens, width = proj.shape[0], rank + rot
+    _need(proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] >= max(q_col + heads * (dim + rot), kv_col + width), "latent_prep: proj rows are too short")
+    _need(pages.dim() == 4 and pages.shape[1] == 1 and pages.shape[3] == width and pages.is_contiguous() and pages.dtype == proj.dtype,
+          f"latent_prep: pages must be contiguous [P, 1, page, {width}] of the rows' dtype")
+    _need(queries.shape == (tokens, heads, width) and queries.is_contiguous() and queries.dtype == proj.dtype, f"latent_prep: queries must be [{tokens}, {heads}, {width}]")
+    _need(norm_weight.numel() == rank and norm_weight.is_contiguous(), f"latent_prep: the norm weight must hold {rank} values")
+    _need(slots.dtype == torch.int32 and slots.numel() >= tokens and slots.is_contiguous(), "latent_prep: slots must be int32 [T]")
+    for name, t in (("cos", cos), ("sin", sin)):
+        _need((t is None) == (cos is None) and (t is None or (t.dtype == torch.float32 and t.shape == (tokens, rot // 2) and t.is_contiguous())),
+              f"latent_prep: {name} must be float32 [{tokens}, {rot // 2}]")
+    _launch("lrs_latent_prep", _dev(proj, "proj"), proj.stride(0), dtype_code(proj.dtype), tokens, q_col, kv_col, heads, dim, rot, rank,
+            _dev(norm_weight, "norm_weight"), dtype_code(norm_weight.dtype), eps, None if cos is None else _dev(cos, "cos"),
+            None if sin is None else _dev(sin, "sin"), _dev(pages, "pages"), _dev(slots, "slots"), _dev(queries, "queries"), heads * width, _stream())
+
+
+def head_gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, transposed: bool) -> None:
+    """out [T, heads, n] = per head h: w[h] a[t, h] with w [heads, n, k], or w[h]^T a[t, h] with w [heads, k, n] if `transposed`.
+    out and a may be views with strides of their own between tokens and heads."""
+    tokens, heads, n = out.shape
+    k = a.shape[2]
+    _need(a.shape[:2] == (tokens, heads) and a.stride(2) == 1 and out.stride(2) == 1 and a.dtype == out.dtype == w.dtype, "head_gemm: a [T, heads, k] and out [T, heads, n] of the weights' dtype")
+    _need(w.is_contiguous() and w.shape == ((heads, k, n) if transposed else (heads, n, k)), f"head_gemm: w must be contiguous [{heads}, {k if transposed else n}, {n if transposed else k}]")
+    _launch("lrs_head_gemm", _dev(out, "out"), out.stride(0), out.stride(1), _dev(a, "a"), a.stride(0), a.stride(1), _dev(w, "w"), n * k, int(transposed),
+            dtype_code(w.dtype), tokens, heads, n, k, _stream())
+
+
+def latent_attention(out: torch.Tensor, queries: torch.Tensor, pages: torch.Tensor, block_table: torch.Tensor, token_request: torch.Tensor,
+                     positions: torch.Tensor, rank: int, scale: float, sink: torch.Tensor | None = None, gate: torch.Tensor | None = None,
+                     window: int = 0) -> None:
+    """out [T, heads * rank] = per (token, head): softmax over the request's kept rows j <= position (within `window` if
+    given) of (queries[t, h] . row_j) * scale, with exp(sink[h]) as one more term of the denominator, times row_j[:rank],
+    times sigmoid(gate[t, h]).  pages [P, 1, page, width]; gate: a [T, heads] view (contiguous along heads)."""
+    tokens, heads, width = queries.shape
+    _need(pages.dim() == 4 and pages.shape[1] == 1 and pages.shape[3] == width and pages.is_contiguous(), f"latent_attention: pages must be contiguous [P, 1, page, {width}]")
+    _need(queries.is_contiguous() and out.shape == (tokens, heads * rank) and out.stride(1) == 1 and 0 < rank <= width, "latent_attention: queries [T, heads, width], out [T, heads * rank]")
+    _need(queries.dtype == pages.dtype == out.dtype, "latent_attention: queries, pages and out must share a dtype")
+    _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.stride(1) == 1, "latent_attention: block_table must be int32 [R, blocks]")
+    for name, t in (("token_request", token_request), ("positions", positions)):
+        _need(t.dtype == torch.int32 and t.numel() >= tokens and t.is_contiguous(), f"latent_attention: {name} must be int32 [T]")
+    _need(sink is None or (sink.dtype == torch.float32 and sink.numel() == heads and sink.is_contiguous()), "latent_attention: sink must hold a float32 per head")
+    _need(gate is None or (gate.shape == (tokens, heads) and gate.stride(1) == 1 and gate.dtype == out.dtype), "latent_attention: gate must be a [T, heads] view of the run's dtype")
+    _launch("lrs_latent_attention", _dev(out, "out"), out.stride(0), _dev(queries, "queries"), heads * width, _dev(pages, "pages"),
+            _dev(block_table, "block_table"), block_table.stride(0), _dev(token_request, "token_request"), _dev(positions, "positions"),
+            None if sink is None else _dev(sink, "sink"), None if gate is None else _dev(gate, "gate"), 0 if gate is None else gate.stride(0),
+            dtype_code(out.dtype), tokens, heads, rank, width, pages.shape[2], scale, window, _stream())

@@ -10,6 +10,11 @@ A sublayer writes its output into a float32 buffer of the step (a part that says
 other adds into the buffer after it has been cleared), and the norm adds the normalised rows into the stream; a
 feed-forward that says `applies_output_norm` is given the norm and does both itself, in the kernel that sums up
 its output.
+
+PostNormBlock: the sublayers read the stream itself and each norm is applied to the sum, which replaces the stream:
+    h = norm1(alpha * h + mixer(h));  h = norm2(alpha * h + feed_forward(h))      (the feed-forward may be absent)
+alpha is a constant of the model.  A sublayer writes into a float32 buffer of the step as for OutputNormBlock, and the norm's
+`scale_add_normed` does the rest in one kernel.
 """
 
 from __future__ import annotations
@@ -200,3 +205,56 @@ class OutputNormBlock(Part):
 
 
 register("block", "outnorm", OutputNormBlock)
+
+
+class PostNormBlock(OutputNormBlock):
+    """h = norm1(alpha * h + mixer(h)); h = norm2(alpha * h + feed_forward(h)).  Everything around the two sums (which
+    buffer a sublayer writes, what is handed to the next block) is OutputNormBlock's."""
+
+    def __init__(self, mixer: PartSpec, mixer_norm: PartSpec, feed_forward: PartSpec | None = None, ff_norm: PartSpec | None = None,
+                 alpha: float = 1.0, names: dict | None = None):
+        if (feed_forward is None) != (ff_norm is None):
+            raise ValueError("a feed-forward and its norm come together")
+        self.alpha = float(alpha)
+        self.mixer = create("mixer", mixer)
+        self.mixer_norm = create("norm", mixer_norm)
+        self.feed_forward = None if feed_forward is None else create("feed_forward", feed_forward)
+        self.ff_norm = None if ff_norm is None else create("norm", ff_norm)
+        for norm in (self.mixer_norm, self.ff_norm):
+            if norm is not None and not callable(getattr(norm, "scale_add_normed", None)):
+                raise ValueError("a norm of the sum of stream and sublayer must offer scale_add_normed(ctx, residual, y, alpha)")
+        self.names = {"mixer": "mixer", "feed_forward": "feed_forward", "mixer_norm": "mixer_norm", "ff_norm": "ff_norm"}
+        self.names.update(names or {})
+
+    def _add_normed(self, ctx, norm, h, y, name):
+        """h = norm(alpha * h + y); returns the new stream as the next reader's activation if the norm's kernel left it."""
+        if ctx.dtype == torch.bfloat16 and getattr(norm, "rounds_stream", False):
+            rounded = ctx.scratch(name, tuple(h.shape), torch.bfloat16)
+            norm.scale_add_normed(ctx, h, y, self.alpha, rounded=rounded)
+            return rounded
+        norm.scale_add_normed(ctx, h, y, self.alpha)
+        return None
+
+    def forward(self, ctx, h, cache, given=None):
+        x = given if given is not None else self._input(ctx, h)
+        y = self._sublayer(ctx, self.mixer, x, h, cache)
+        if self.feed_forward is None:
+            return self._add_normed(ctx, self.mixer_norm, h, y, "stream_rounded_next")
+        x = self._add_normed(ctx, self.mixer_norm, h, y, "stream_rounded_mid")
+        if x is None:
+            x = self._input(ctx, h)
+        y = self._sublayer(ctx, self.feed_forward, x, h)
+        return self._add_normed(ctx, self.ff_norm, h, y, "stream_rounded_next")
+
+    def _sublayer(self, ctx, part, x, h, *cache):
+        """What `part` gives out for the input x, in the step's float32 buffer for sublayer outputs."""
+        if getattr(part, "can_overwrite", False):
+            y = ctx.scratch("sublayer_out", tuple(h.shape), torch.float32)
+            part.forward(ctx, x, y, *cache, accumulate=False)
+        else:
+            y = self._cleared(ctx, h)
+            part.forward(ctx, x, y, *cache)
+        return y
+
+
+register("block", "postnorm", PostNormBlock)

@@ -1,0 +1,138 @@
+"""Latent attention: causal attention whose keys and values are all made from one small row per position.
+
+With h the mixer's input, H heads, per head `dim` plain and `rot` rotated query/key dims, values of `vdim`, a latent row
+of `rank` values:
+
+    q = W_q h                        per head [dim plain | rot rotated]
+    [c_raw | kr_raw] = W_dkv h       rank + rot values
+    c = rms_norm(c_raw) * w_c        the latent row;   kr = rotate(kr_raw), one rotated key part shared by all heads
+    key of head n    = [W_uk[n] c | kr],   value of head n = W_uv[n] c
+    score            = (q_plain . key_plain + rotate(q_rot) . kr) * scale          causal: position i sees j <= i
+    weights          = exp(score) / (sum over j of exp(score) + exp(sink[n]))      the sink has no key and no value
+    out              = W_o concat over n of sigmoid(W_g h)[n] * sum_j weights_j value_j
+
+Only [c | kr] is kept, one row a position (a paged need without value pages).  W_uk and W_uv never meet the kept rows:
+since q_plain . (W_uk[n] c) = (W_uk[n]^T q_plain) . c and sum_j w_j W_uv[n] c_j = W_uv[n] sum_j w_j c_j, the query is carried
+into the latent dims before the attention kernel and its result out of them after, both as small products per (token, head),
+and the kernel attends over the rows as they are kept, all heads reading the same ones.  The gate, one number a head, is
+applied to the latent sum inside the attention kernel.
+
+q, dkv and g are one stacked product.  Norm, rotation, scores, weights and sums are float32 in every precision mode.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from ..kernels import ops
+from .base import PagedKVNeed, Part, PartSpec, TensorSpec, create, register
+from .linear import linear, materialize, rows_of
+
+
+class LatentAttention(Part):
+    graph_safe = True
+    plan_safe = True
+    can_overwrite = True        # forward(..., accumulate=False) stores its output
+
+    def __init__(self, hidden_size: int, num_heads: int, head_dim: int, rot_dim: int, value_dim: int, kv_rank: int, *,
+                 position: PartSpec = PartSpec("none"), norm_eps: float = 1e-6, scale: float | None = None, sink: bool = False,
+                 gate: bool = False, window: int | None = None):
+        for name, value in (("hidden_size", hidden_size), ("num_heads", num_heads), ("head_dim", head_dim), ("value_dim", value_dim), ("kv_rank", kv_rank)):
+            if value <= 0:
+                raise ValueError(f"{name} must be positive, got {value}")
+        if rot_dim < 0 or rot_dim % 2:
+            raise ValueError(f"rot_dim must be even and not negative, got {rot_dim}")
+        if scale is not None and (not math.isfinite(scale) or scale <= 0):
+            raise ValueError(f"scale must be finite and positive, got {scale}")
+        if window is not None and window <= 0:
+            raise ValueError(f"window must be positive when given, got {window}")
+        if norm_eps <= 0:
+            raise ValueError(f"norm_eps must be positive, got {norm_eps}")
+        self.hidden_size, self.num_heads, self.head_dim, self.rot_dim = hidden_size, num_heads, head_dim, rot_dim
+        self.value_dim, self.kv_rank, self.norm_eps, self.window = value_dim, kv_rank, norm_eps, window
+        self.position = create("position", position)
+        if getattr(self.position, "rotary_dim", rot_dim) != rot_dim:
+            raise ValueError(f"the position part rotates {self.position.rotary_dim} dims, the mixer's rotated part has {rot_dim}")
+        self.scale = 1.0 / math.sqrt(head_dim + rot_dim) if scale is None else scale
+        self.has_sink, self.has_gate = sink, gate
+        self.w_in = self.w_uk = self.w_uv = self.w_o = self.latent_norm = self.sink = None
+
+    # ------------------------------------------------------------------ weights
+    @property
+    def width(self) -> int:
+        """Values kept per position."""
+        return self.kv_rank + self.rot_dim
+
+    def tensors(self):
+        h, n, r = self.hidden_size, self.num_heads, self.kv_rank
+        specs = {
+            "q_proj.weight": TensorSpec((n * (self.head_dim + self.rot_dim), h)),
+            "dkv_proj.weight": TensorSpec((self.width, h)),
+            "dkv_norm.weight": TensorSpec((r,), role="norm"),
+            "uk_proj.weight": TensorSpec((n * self.head_dim, r)),
+            "uv_proj.weight": TensorSpec((n * self.value_dim, r)),
+            "o_proj.weight": TensorSpec((h, n * self.value_dim)),
+        }
+        if self.has_sink:
+            specs["sink"] = TensorSpec((n,), role="bias")
+        if self.has_gate:
+            specs["g_proj.weight"] = TensorSpec((n, h))
+        return specs
+
+    def bind(self, weights, dtype):
+        n = self.num_heads
+        stacked = [weights["q_proj.weight"], weights["dkv_proj.weight"]] + ([weights["g_proj.weight"]] if self.has_gate else [])
+        w_in = torch.cat(stacked, 0).to(dtype)
+        pad = -w_in.shape[0] % 16             # whole groups of 16 output columns suit every product kernel
+        if pad:
+            w_in = torch.cat((w_in, w_in.new_zeros(pad, self.hidden_size)), 0)
+        self.w_in = w_in.contiguous()
+        self.kv_col = n * (self.head_dim + self.rot_dim)
+        self.gate_col = self.kv_col + self.width
+        self.w_uk = weights["uk_proj.weight"].to(dtype).reshape(n, self.head_dim, self.kv_rank).contiguous()
+        self.w_uv = weights["uv_proj.weight"].to(dtype).reshape(n, self.value_dim, self.kv_rank).contiguous()
+        self.w_o = weights["o_proj.weight"].to(dtype).contiguous()
+        self.latent_norm = weights["dkv_norm.weight"]
+        self.sink = weights["sink"].float().contiguous() if self.has_sink else None
+
+    def weight_bytes(self):
+        return (self.w_in.numel() + self.w_uk.numel() + self.w_uv.numel() + self.w_o.numel()) * self.w_o.element_size()
+
+    def flops(self, tokens, pairs):
+        if self.window is not None:
+            pairs = min(pairs, tokens * self.window)
+        # the projections (the two per-head ones count their matrices once a token, as the others), then scores over the
+        # kept rows and the weighted sum of their latent part, per pair and head
+        return super().flops(tokens, pairs) + 2.0 * pairs * self.num_heads * (self.width + self.kv_rank)
+
+    def cache_need(self):
+        return PagedKVNeed(1, self.width, self.window, values=False)
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, ctx, x, residual, cache, then_norm=None, accumulate: bool = True):
+        if cache is None:
+            raise ValueError("latent attention needs a paged cache")
+        t, n, r = rows_of(x), self.num_heads, self.kv_rank
+        x = materialize(ctx, x)
+        group = ctx.group(cache.group)
+        proj = ctx.scratch("latent_proj", (t, self.w_in.shape[0]), ctx.dtype)
+        linear(ctx, proj, x, self.w_in)
+        tables = self.position.tables(ctx) if self.rot_dim else None
+        cos, sin = tables if tables is not None else (None, None)
+        queries = ctx.scratch("latent_queries", (t, n, self.width), ctx.dtype)
+        ops.latent_prep(proj, 0, self.kv_col, n, self.head_dim, self.rot_dim, r, self.latent_norm, self.norm_eps, cos, sin,
+                        cache.k_pages, group.slots, queries)
+        plain = proj[:, :self.kv_col].view(t, n, self.head_dim + self.rot_dim)[:, :, :self.head_dim]
+        ops.head_gemm(queries[:, :, :r], plain, self.w_uk, transposed=True)
+        latent = ctx.scratch("latent_out", (t, n * r), ctx.dtype)
+        gate = proj[:, self.gate_col:self.gate_col + n] if self.has_gate else None
+        ops.latent_attention(latent, queries, cache.k_pages, group.block_table, ctx.token_slot, ctx.positions, r, self.scale,
+                             sink=self.sink, gate=gate, window=self.window or 0)
+        heads_out = ctx.scratch("latent_heads_out", (t, n, self.value_dim), ctx.dtype)
+        ops.head_gemm(heads_out, latent.view(t, n, r), self.w_uv, transposed=False)
+        return linear(ctx, residual, heads_out.view(t, n * self.value_dim), self.w_o, accumulate=accumulate, then_norm=then_norm)
+
+
+register("mixer", "latent_attention", LatentAttention)

@@ -2,7 +2,7 @@
 
 Reference mini_llm/nn/mlp.py:80-87.  gate and up are stacked into one [2I, H] matrix when
 the weights are bound, so one product feeds the gated activation; the down projection adds
-straight into the float32 residual stream.
+straight into the float32 residual stream (or, with `accumulate=False`, stores into the float32 rows it is given).
 """
 
 from __future__ import annotations
@@ -19,6 +19,7 @@ class SwiGLU(Part):
     plan_safe = True
     takes_lazy_norm = True
     begins_next_norm = True
+    can_overwrite = True        # forward(..., accumulate=False) stores its output
 
     def __init__(self, hidden_size: int, intermediate_size: int):
         if hidden_size <= 0 or intermediate_size <= 0:
@@ -50,7 +51,7 @@ class SwiGLU(Part):
     def weight_bytes(self):
         return (self.gate_up.numel() + self.down.numel()) * self.down.element_size()
 
-    def forward(self, ctx, x, residual, then_norm=None):
+    def forward(self, ctx, x, residual, then_norm=None, accumulate: bool = True):
         t = rows_of(x)
         act = ctx.scratch("ffn_act", (t, self.intermediate_size), ctx.dtype)
         if self.interleaved:
@@ -59,7 +60,7 @@ class SwiGLU(Part):
             gate_up = ctx.scratch("ffn_gate_up", (t, 2 * self.intermediate_size), ctx.dtype)
             linear(ctx, gate_up, x, self.gate_up)
             ops.silu_mul(act, gate_up)
-        return linear(ctx, residual, act, self.down, accumulate=True, then_norm=then_norm)
+        return linear(ctx, residual, act, self.down, accumulate=accumulate, then_norm=then_norm)
 
 
 register("feed_forward", "swiglu", SwiGLU)

@@ -1,8 +1,12 @@
 """Routed experts: a feed-forward made of many small ones, of which every token runs a few.
 
-    z = W_router x (+ bias)                        float32 (x may be the activation's rounding)
-    chosen = the `top` largest z;  p = softmax(z[chosen])
-    out = sum over chosen e of p_e * W_down_e act(W_up_e x)         act: the square of relu, or relu
+    z = W_router x                                 float32 (x may be the activation's rounding)
+    rule "softmax_chosen":  chosen = the `top` largest z + bias;  p = softmax((z + bias)[chosen])
+    rule "sigmoid":         s = sigmoid(z); chosen = the `top` largest s + bias (the bias takes part in the choice only;
+                            with groups, among the experts of the `keep` groups whose two largest s + bias sum highest);
+                            p = s[chosen] / (sum of s[chosen] + 1e-20) * scale
+    out = sum over chosen e of p_e * expert_e(x)
+    expert "relu_squared":  W_down relu(W_up x)^2;   "silu_gated":  W_down (silu(W_gate x) * (W_up x))
 
 On the device: the router product, the choice per token, one sort of the step's (token, choice) pairs by expert
 into runs padded to whole row tiles, two grouped products over the sorted rows (the activation in the first one's
@@ -19,7 +23,7 @@ from ..kernels import ops
 from .base import Part, TensorSpec, register
 from .linear import kernels_of, materialize, rows_of, workspace_of
 
-ACTIVATIONS = ("relu_squared",)
+ACTIVATIONS = ("relu_squared", "silu_gated")
 
 
 class RoutedExperts(Part):
@@ -29,7 +33,8 @@ class RoutedExperts(Part):
     rounds_stream = True          # forward(..., rounded=buffer): the updated stream is left there in bfloat16 as well
 
     def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int, top: int, router_bias: bool = False,
-                 activation: str = "relu_squared"):
+                 activation: str = "relu_squared", rule: str = "softmax_chosen", groups: int = 0, keep: int = 0, weight_scale: float = 1.0,
+                 bias_name: str = "router.bias"):
         if min(hidden_size, intermediate_size, num_experts, top) <= 0:
             raise ValueError("hidden_size, intermediate_size, num_experts and top must be positive")
         if top > num_experts:
@@ -39,15 +44,25 @@ class RoutedExperts(Part):
         if activation not in ACTIVATIONS:
             raise ValueError(f"unknown activation {activation!r}; known: {', '.join(ACTIVATIONS)}")
         self.hidden_size, self.intermediate_size, self.num_experts, self.top = hidden_size, intermediate_size, num_experts, top
-        self.router_bias, self.activation = router_bias, activation
+        self.router_bias, self.activation, self.bias_name = router_bias, activation, bias_name
+        self.rule = ops.RouteRule(rule, groups, keep, weight_scale)
+        if rule not in ops.RouteRule.KINDS:
+            raise ValueError(f"unknown routing rule {rule!r}; known: {', '.join(ops.RouteRule.KINDS)}")
+        if groups and (rule != "sigmoid" or num_experts % groups or not 0 < keep <= groups or keep * (num_experts // groups) < top):
+            raise ValueError(f"{num_experts} experts in {groups} groups of which {keep} are kept cannot give {top} choices under rule {rule!r}")
+        if not weight_scale > 0:
+            raise ValueError(f"weight_scale must be positive, got {weight_scale}")
+        self.gated = activation == "silu_gated"
         self.router = self.bias = self.up = self.down = None
 
     def tensors(self):
         h, i = self.hidden_size, self.intermediate_size
         specs = {"router.weight": TensorSpec((self.num_experts, h))}
         if self.router_bias:
-            specs["router.bias"] = TensorSpec((self.num_experts,), role="bias")
+            specs[self.bias_name] = TensorSpec((self.num_experts,), role="bias")
         for e in range(self.num_experts):
+            if self.gated:
+                specs[f"experts.{e}.gate.weight"] = TensorSpec((i, h))
             specs[f"experts.{e}.up.weight"] = TensorSpec((i, h))
             specs[f"experts.{e}.down.weight"] = TensorSpec((h, i))
         return specs
@@ -58,17 +73,21 @@ class RoutedExperts(Part):
         if pad:
             router = torch.cat((router, router.new_zeros(pad, self.hidden_size)), 0)
         self.router = router.contiguous()
-        self.bias = weights["router.bias"].float().contiguous() if self.router_bias else None
-        self.up = torch.stack([weights[f"experts.{e}.up.weight"].to(dtype) for e in range(self.num_experts)]).contiguous()
+        self.bias = weights[self.bias_name].float().contiguous() if self.router_bias else None
+        if self.gated:      # an expert's gate rows, then its up rows: one product makes both
+            self.up = torch.stack([torch.cat((weights[f"experts.{e}.gate.weight"], weights[f"experts.{e}.up.weight"]), 0).to(dtype)
+                                   for e in range(self.num_experts)]).contiguous()
+        else:
+            self.up = torch.stack([weights[f"experts.{e}.up.weight"].to(dtype) for e in range(self.num_experts)]).contiguous()
         self.down = torch.stack([weights[f"experts.{e}.down.weight"].to(dtype) for e in range(self.num_experts)]).contiguous()
 
     def weight_bytes(self):
         """What a decode step of one token reads: the router and the chosen experts."""
-        chosen = 2 * self.top * self.hidden_size * self.intermediate_size
+        chosen = (3 if self.gated else 2) * self.top * self.hidden_size * self.intermediate_size
         return (self.router.numel() + chosen) * self.up.element_size()
 
     def flops(self, tokens, pairs):
-        return 2.0 * tokens * (self.num_experts * self.hidden_size + 2 * self.top * self.hidden_size * self.intermediate_size)
+        return 2.0 * tokens * (self.num_experts * self.hidden_size + (3 if self.gated else 2) * self.top * self.hidden_size * self.intermediate_size)
 
     def forward(self, ctx, x, residual, then_norm=None, output_norm=None, rounded=None):
         t = rows_of(x)
@@ -84,12 +103,17 @@ class RoutedExperts(Part):
         place = ctx.scratch("moe_place", (t * top,), torch.int32)
         tile_expert = ctx.scratch("moe_tile_expert", (tiles,), torch.int32)
         if t <= ops.ROUTE_ALIGN_TOKENS:        # few tokens: the choice and the sort in one launch
-            ops.moe_route_align(logits[:, :experts], self.bias, ids, weights, sorted_pairs, place, tile_expert)
+            ops.moe_route_align(logits[:, :experts], self.bias, ids, weights, sorted_pairs, place, tile_expert, rule=self.rule)
         else:
-            ops.moe_route(logits[:, :experts], self.bias, ids, weights)
+            ops.moe_route(logits[:, :experts], self.bias, ids, weights, rule=self.rule)
             ops.moe_align(ids, experts, sorted_pairs, place, tile_expert)
         hidden = ctx.scratch("moe_hidden", (rows, self.intermediate_size), ctx.dtype)
-        ops.moe_experts(hidden, x, self.up, sorted_pairs, tile_expert, tile, top, gather=True, relu_squared=True)
+        if self.gated:
+            both = ctx.scratch("moe_gate_up", (rows, 2 * self.intermediate_size), ctx.dtype)
+            ops.moe_experts(both, x, self.up, sorted_pairs, tile_expert, tile, top, gather=True, relu_squared=False)
+            ops.silu_mul(hidden, both)
+        else:
+            ops.moe_experts(hidden, x, self.up, sorted_pairs, tile_expert, tile, top, gather=True, relu_squared=True)
         outputs = ctx.scratch("moe_outputs", (rows, self.hidden_size), torch.float32)
         ops.moe_experts(outputs, hidden, self.down, sorted_pairs, tile_expert, tile, top, gather=False, relu_squared=False)
         if output_norm is None:

@@ -61,3 +61,42 @@ class RMSNorm(Part):
 
 
 register("norm", "rmsnorm", RMSNorm)
+
+
+class LayerNorm(Part):
+    """y = w * (x - mean) / sqrt(variance + eps) over the last dimension, the variance being the mean of the squared
+    deviations; a weight and no bias.  Statistics in float32, one rounding at the output.
+
+    Besides `forward` it serves layer arrangements that normalise the sum of the stream and a sublayer's output
+    (parts/block.py, PostNormBlock): `scale_add_normed(ctx, residual, y, alpha)` replaces the stream by the norm of
+    alpha * stream + y."""
+
+    graph_safe = True
+    plan_safe = True
+    rounds_stream = True   # scale_add_normed(..., rounded=buffer) also leaves the new rows in bfloat16
+
+    def __init__(self, size: int, eps: float):
+        if size <= 0:
+            raise ValueError(f"size must be positive, got {size}")
+        if eps <= 0:
+            raise ValueError(f"eps must be positive, got {eps}")
+        self.size, self.eps = size, eps
+        self.weight = None
+
+    def tensors(self):
+        return {"weight": TensorSpec((self.size,), role="norm")}
+
+    def bind(self, weights, dtype):
+        self.weight = weights["weight"]
+
+    def scale_add_normed(self, ctx, residual, y, alpha: float, rounded=None):
+        ops.scale_add_layernorm(residual, y, alpha, self.weight, self.eps, rounded)
+
+    def forward(self, ctx, h, rows=None, count=None):
+        n = h.shape[0] if rows is None else count
+        out = ctx.scratch("norm_out", (n, h.shape[1]), ctx.dtype)
+        ops.layernorm(out, h, self.weight, self.eps, rows=rows)
+        return out
+
+
+register("norm", "layernorm", LayerNorm)
