@@ -31,3 +31,20 @@ def nobodra_like(shape: dict, layers: int, experts: int = 32, top: int = 8, wind
     delta = {"type": "delta", "mlp": mlp, "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "conv": 4}}
     return {"architecture": "Nobodra", "vocab": shape["vocab_size"], "width": width, "norm": {"eps": 1e-6},
             "layers": [attention if index % 4 == 3 else delta for index in range(layers)]}
+
+
+def napizen_like(shape: dict, layers: int, experts: int = 32, top: int = 8, rank: int = 512, rot: int = 64) -> dict:
+    """A Napizen configuration with the layer sizes of a dense shape above, for measurements beside it: the same width,
+    vocabulary and number of heads; heads of the shape's size plain and `rot` rotated dims, values of the shape's head size,
+    `rank` latent values a position; layers with the dense feed-forward of the shape's `intermediate_size` in turn with layers
+    of `top` of `experts` gated experts with as many weights in use per token (to a multiple of 128), chosen among half of
+    eight groups."""
+    width, heads, dim = shape["hidden_size"], shape["num_attention_heads"], shape["head_dim"]
+    ff = max(128, round(shape["intermediate_size"] / top / 128) * 128)
+    mixer = {"heads": heads, "dim": dim, "rot_dim": rot, "vdim": dim, "kv_rank": rank, "scale": (dim + rot) ** -0.5,
+             "rot": {"base": 1000000.0, "dims": rot, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+    dense = {"kind": "dense", "ff": shape["intermediate_size"]}
+    routed = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top, "scale": 2.5, "groups": {"count": 8, "keep": 4}}}
+    return {"architecture": "Napizen", "vocab": shape["vocab_size"], "width": width, "norm": {"eps": 1e-6}, "postln_alpha": 2.0,
+            "embedding": {"scale": 1.0}, "logit_softcap": 30.0,
+            "layers": [{"type": "latent_attention", "mixer": mixer, "mlp": routed if index % 2 else dense} for index in range(layers)]}

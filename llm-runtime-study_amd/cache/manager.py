@@ -2,8 +2,8 @@
 fixed-size per-request state.
 
 What each schedule entry of the model keeps between steps is declared by its mixer:
-  PagedKVNeed(nkv, d, window, dtype, values)  keys and values of every position, or of a sliding window, kept in `dtype`
-                               (None: the run's activation dtype); values False: key pages alone (one row a position);
+  PagedKVNeed(nkv, d, window, dtype, value_dim)  keys and values of every position, or of a sliding window, kept in `dtype`
+                               (None: the run's activation dtype); value_dim: rows of a value page if not d, 0: key pages alone;
   StateNeed(shape, dtype)      a state of fixed size;
   ("from", j)                  nothing of its own: it reads the cache of entry j;
   None                         nothing.
@@ -151,11 +151,12 @@ class CacheManager:
         for index, group in enumerate(self.groups):
             if allocate_storage:
                 k_shape = (num_pages + 1, group.need.num_kv_heads, page_size, group.need.head_dim)
-                v_shape = (num_pages + 1, group.need.num_kv_heads, group.need.head_dim, page_size)
+                value_dim = group.need.head_dim if group.need.value_dim is None else group.need.value_dim
+                v_shape = (num_pages + 1, group.need.num_kv_heads, value_dim, page_size)
                 for position in group.entries:
                     group.k[position] = torch.zeros(k_shape, dtype=group.dtype, device=self.device)
                     self.layer_caches[position].k_pages = group.k[position]
-                    if group.need.values:
+                    if value_dim:
                         group.v[position] = torch.zeros(v_shape, dtype=group.dtype, device=self.device)
                         self.layer_caches[position].v_pages = group.v[position]
 
@@ -184,8 +185,8 @@ class CacheManager:
         return max((g.pool.used_pages for g in self.groups), default=0) * self.page_size
 
     def bytes_per_token(self) -> int:
-        return sum((2 if g.need.values else 1) * len(g.entries) * g.need.num_kv_heads * g.need.head_dim * torch.empty(0, dtype=g.dtype).element_size()
-                   for g in self.groups)
+        return sum(len(g.entries) * g.need.num_kv_heads * (g.need.head_dim + (g.need.head_dim if g.need.value_dim is None else g.need.value_dim))
+                   * torch.empty(0, dtype=g.dtype).element_size() for g in self.groups)
 
     def trash_page(self, group: int = 0) -> int:
         """Page that no request owns; padding rows of a padded batch write there."""

@@ -161,7 +161,11 @@ _SIGNATURES = {
     "lrs_scale_add_layernorm": (c_int, [c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_int, c_float, c_void_p, c_void_p]),
     "lrs_soft_cap": (c_int, [c_void_p, c_int64, c_float, c_void_p]),
     "lrs_latent_prep": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p,
-                                c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+                                c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p]),
+    "lrs_latent_attention_groups_takes": (c_int, [c_int, c_int, c_int]),
+    "lrs_latent_attention_groups": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                                            c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
+                                            c_void_p, c_void_p, c_void_p]),
     "lrs_head_gemm": (c_int, [c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "lrs_latent_attention": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                      c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
@@ -204,7 +208,7 @@ def library():
 PLAN_OPS = ("lrs_add_into", "lrs_add_rmsnorm", "lrs_advance_decode", "lrs_advance_slots", "lrs_attention", "lrs_attention_decode",
             "lrs_attention_prefill", "lrs_choose_tokens", "lrs_choose_tokens_split", "lrs_copy_to_pinned", "lrs_delta_rule", "lrs_embed", "lrs_fill_i32",
             "lrs_filter_logits", "lrs_gather_rows", "lrs_gemm", "lrs_gemm_lines_add_rmsnorm", "lrs_gemm_mid_add_norm_begin", "lrs_gemm_mid_qk_prep", "lrs_gemm_mid_scaled",
-            "lrs_gemm_norm_chain", "lrs_head_gemm", "lrs_latent_attention", "lrs_latent_prep", "lrs_layernorm", "lrs_library_gemm", "lrs_moe_align", "lrs_moe_combine", "lrs_moe_experts", "lrs_moe_route", "lrs_moe_route_align", "lrs_norm_add",
+            "lrs_gemm_norm_chain", "lrs_head_gemm", "lrs_latent_attention", "lrs_latent_attention_groups", "lrs_latent_prep", "lrs_layernorm", "lrs_library_gemm", "lrs_moe_align", "lrs_moe_combine", "lrs_moe_experts", "lrs_moe_route", "lrs_moe_route_align", "lrs_norm_add",
             "lrs_qk_prep", "lrs_rmsnorm", "lrs_rope_table", "lrs_round_rows", "lrs_scale_add_layernorm", "lrs_scale_rows", "lrs_silu_mul", "lrs_soft_cap")
 _PLAN_INDEX = {name: index for index, name in enumerate(PLAN_OPS)}
 
@@ -1330,16 +1334,20 @@ def moe_combine(residual: torch.Tensor, rows: torch.Tensor, place: torch.Tensor,
 
 # ------------------------------------------------------------------- latent attention
 def latent_prep(proj: torch.Tensor, q_col: int, kv_col: int, heads: int, dim: int, rot: int, rank: int, norm_weight: torch.Tensor, eps: float,
-                cos: torch.Tensor | None, sin: torch.Tensor | None, pages: torch.Tensor, slots: torch.Tensor, queries: torch.Tensor) -> None:
+                cos: torch.Tensor | None, sin: torch.Tensor | None, pages: torch.Tensor, slots: torch.Tensor, queries: torch.Tensor,
+                value_pages: torch.Tensor | None = None) -> None:
     """Per token of proj [T, columns]: the RMS norm (norm_weight, eps) of the `rank` latent values at column kv_col and the
     rotation (pairs 2i, 2i + 1; cos, sin [T, rot / 2], None: none) of the `rot` shared key values behind them, written into
     the token's row of pages [P, 1, page, rank + rot] (slots[t] < 0: not kept); and the rotation of the last `rot` of the
-    dim + rot values of every head's query (from column q_col on) into queries [T, heads, rank + rot][..., rank:]."""
+    dim + rot values of every head's query (from column q_col on) into queries [T, heads, rank + rot][..., rank:].
+    value_pages [P, 1, rank, page]: receives the normed latent values as well, transposed inside a page."""
     tokens, width = proj.shape[0], rank + rot
     _need(proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] >= max(q_col + heads * (dim + rot), kv_col + width), "latent_prep: proj rows are too short")
     _need(pages.dim() == 4 and pages.shape[1] == 1 and pages.shape[3] == width and pages.is_contiguous() and pages.dtype == proj.dtype,
           f"latent_prep: pages must be contiguous [P, 1, page, {width}] of the rows' dtype")
     _need(queries.shape == (tokens, heads, width) and queries.is_contiguous() and queries.dtype == proj.dtype, f"latent_prep: queries must be [{tokens}, {heads}, {width}]")
+    _need(value_pages is None or (value_pages.shape == (pages.shape[0], 1, rank, pages.shape[2]) and value_pages.is_contiguous() and value_pages.dtype == pages.dtype),
+          f"latent_prep: value pages must be contiguous [P, 1, {rank}, page] of the pages' dtype")
     _need(norm_weight.numel() == rank and norm_weight.is_contiguous(), f"latent_prep: the norm weight must hold {rank} values")
     _need(slots.dtype == torch.int32 and slots.numel() >= tokens and slots.is_contiguous(), "latent_prep: slots must be int32 [T]")
     for name, t in (("cos", cos), ("sin", sin)):
@@ -1347,7 +1355,8 @@ def latent_prep(proj: torch.Tensor, q_col: int, kv_col: int, heads: int, dim: in
               f"latent_prep: {name} must be float32 [{tokens}, {rot // 2}]")
     _launch("lrs_latent_prep", _dev(proj, "proj"), proj.stride(0), dtype_code(proj.dtype), tokens, q_col, kv_col, heads, dim, rot, rank,
             _dev(norm_weight, "norm_weight"), dtype_code(norm_weight.dtype), eps, None if cos is None else _dev(cos, "cos"),
-            None if sin is None else _dev(sin, "sin"), _dev(pages, "pages"), _dev(slots, "slots"), _dev(queries, "queries"), heads * width, _stream())
+            None if sin is None else _dev(sin, "sin"), _dev(pages, "pages"), None if value_pages is None else _dev(value_pages, "value_pages"), pages.shape[2],
+            _dev(slots, "slots"), _dev(queries, "queries"), heads * width, _stream())
 
 
 def head_gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, transposed: bool) -> None:
@@ -1380,3 +1389,47 @@ def latent_attention(out: torch.Tensor, queries: torch.Tensor, pages: torch.Tens
             _dev(block_table, "block_table"), block_table.stride(0), _dev(token_request, "token_request"), _dev(positions, "positions"),
             None if sink is None else _dev(sink, "sink"), None if gate is None else _dev(gate, "gate"), 0 if gate is None else gate.stride(0),
             dtype_code(out.dtype), tokens, heads, rank, width, pages.shape[2], scale, window, _stream())
+
+
+def latent_attention_groups_takes(dtype: torch.dtype, rank: int, width: int, page_size: int) -> bool:
+    """Whether latent_attention_groups() takes the shape (else latent_attention())."""
+    return dtype == torch.bfloat16 and bool(library().lrs_latent_attention_groups_takes(rank, width, page_size))
+
+
+def latent_attention_groups(out: torch.Tensor, queries: torch.Tensor, pages: torch.Tensor, value_pages: torch.Tensor, block_table: torch.Tensor,
+                            token_request: torch.Tensor, positions: torch.Tensor, group_token0: torch.Tensor | None, group_count: torch.Tensor | None,
+                            max_count: int, rank: int, scale: float, sink: torch.Tensor | None = None, gate: torch.Tensor | None = None, window: int = 0,
+                            splits: int = 1, part_o: torch.Tensor | None = None, part_ml: torch.Tensor | None = None) -> None:
+    """latent_attention() on the matrix cores, bfloat16.  group_token0 / group_count list groups of at most max_count consecutive
+    tokens of one request that together cover every token once (both None: every token alone); value_pages [P, 1, rank, page]
+    holds the latent values once more, transposed inside a page.  splits > 1 divides every group's keys between that many
+    workgroups; their results meet in part_o [T, heads * splits * rank] and part_ml [T, heads * splits * 2] float32."""
+    tokens, heads, width = queries.shape
+    page_size = pages.shape[2]
+    _need(pages.dim() == 4 and pages.shape[1] == 1 and pages.shape[3] == width and pages.is_contiguous(), f"latent_attention_groups: pages must be contiguous [P, 1, page, {width}]")
+    _need(value_pages.shape == (pages.shape[0], 1, rank, page_size) and value_pages.is_contiguous(), f"latent_attention_groups: value pages must be contiguous [P, 1, {rank}, page]")
+    _need(latent_attention_groups_takes(queries.dtype, rank, width, page_size), f"latent_attention_groups: unsupported shape rank={rank} width={width} page={page_size} {queries.dtype}")
+    _need(queries.is_contiguous() and out.shape == (tokens, heads * rank) and out.stride(1) == 1, "latent_attention_groups: queries [T, heads, width], out [T, heads * rank]")
+    _need(queries.dtype == pages.dtype == value_pages.dtype == out.dtype, "latent_attention_groups: queries, pages and out must share a dtype")
+    _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.stride(1) == 1, "latent_attention_groups: block_table must be int32 [R, blocks]")
+    for name, t in (("token_request", token_request), ("positions", positions)):
+        _need(t.dtype == torch.int32 and t.numel() >= tokens and t.is_contiguous(), f"latent_attention_groups: {name} must be int32 [T]")
+    groups = tokens
+    if group_token0 is not None or group_count is not None:
+        groups = group_token0.numel()
+        _need(groups > 0 and group_count.numel() == groups and group_token0.dtype == group_count.dtype == torch.int32 and group_token0.is_contiguous()
+              and group_count.is_contiguous(), "latent_attention_groups: the groups must be two int32 vectors of one length")
+    else:
+        _need(max_count == 1, "latent_attention_groups: tokens without groups stand alone")
+    _need(sink is None or (sink.dtype == torch.float32 and sink.numel() == heads and sink.is_contiguous()), "latent_attention_groups: sink must hold a float32 per head")
+    _need(gate is None or (gate.shape == (tokens, heads) and gate.stride(1) == 1 and gate.dtype == out.dtype), "latent_attention_groups: gate must be a [T, heads] view of the run's dtype")
+    _need(1 <= splits <= 64, f"latent_attention_groups: splits must be 1..64, got {splits}")
+    if splits > 1:
+        _need(part_o is not None and part_o.dtype == torch.float32 and part_o.is_contiguous() and part_o.numel() >= tokens * heads * splits * rank, "latent_attention_groups: part_o too small")
+        _need(part_ml is not None and part_ml.dtype == torch.float32 and part_ml.is_contiguous() and part_ml.numel() >= tokens * heads * splits * 2, "latent_attention_groups: part_ml too small")
+    _launch("lrs_latent_attention_groups", _dev(out, "out"), out.stride(0), _dev(queries, "queries"), heads * width, _dev(pages, "pages"),
+            _dev(value_pages, "value_pages"), _dev(block_table, "block_table"), block_table.stride(0), _dev(token_request, "token_request"),
+            _dev(positions, "positions"), None if group_token0 is None else _dev(group_token0, "group_token0"),
+            None if group_count is None else _dev(group_count, "group_count"), groups, max_count, None if sink is None else _dev(sink, "sink"),
+            None if gate is None else _dev(gate, "gate"), 0 if gate is None else gate.stride(0), tokens, heads, rank, width, page_size, scale, window,
+            splits, None if splits == 1 else _dev(part_o, "part_o"), None if splits == 1 else _dev(part_ml, "part_ml"), _stream())

@@ -185,14 +185,15 @@ class TensorSpec:
 @dataclass(frozen=True)
 class PagedKVNeed:
     """A mixer that keeps keys and values of every position (or of a window) in pages; `dtype`: what the pages
-    hold, if not the run's activation dtype.  `values` False: one row a position and kv head only (the key pages); a
-    mixer whose values are read out of what its keys are made of keeps no second tensor."""
+    hold, if not the run's activation dtype.  `value_dim`: rows of the value pages, [pages, kv heads, value_dim, page] (None: as
+    many as head_dim); 0: no value pages at all, one row a position and kv head only (a mixer whose values are read out of
+    what its keys are made of needs no second tensor)."""
 
     num_kv_heads: int
     head_dim: int
     window: int | None = None
     dtype: torch.dtype | None = None
-    values: bool = True
+    value_dim: int | None = None
 
 
 @dataclass(frozen=True)

@@ -40,8 +40,8 @@ def test_configuration_reads_back_and_names_its_tensors(tmp_path):
                 assert names[f"{p}mlp.e{last}.gate"].shape == (mlp["expert"]["ff"], raw["width"]) and names[f"{p}mlp.e0.down"].shape == (raw["width"], mlp["expert"]["ff"])
                 assert names[p + "mlp.router"].shape == (last + 1, raw["width"]) and names[p + "mlp.correction"].shape == (last + 1,)
         for layer, need in zip(raw["layers"], model.cache_needs()):
-            # one row a position: the latent values and the shared rotated key part, and no value pages
-            assert need == PagedKVNeed(1, layer["mixer"]["kv_rank"] + layer["mixer"]["rot_dim"], None, values=False)
+            # one row a position: the latent values and the shared rotated key part, and no value pages (an unbound model)
+            assert need == PagedKVNeed(1, layer["mixer"]["kv_rank"] + layer["mixer"]["rot_dim"], None, value_dim=0)
         assert model.graph_safe() and model.plan_safe()
     folder = configs.write_folder(configs.MIXED, 3, tmp_path / "m")
     assert load_config(folder).to_json_dict() == configs.MIXED
