@@ -244,6 +244,7 @@ __global__ __launch_bounds__(256) void head_gemm_bf16_kernel(bf16* __restrict__ 
 // they take.  The four waves of a workgroup read the same keys.  Key tiles start at multiples of 32 from position 0.  With
 // splits > 1 a workgroup walks one part of the tiles and leaves its maximum, sum and unscaled output for the merge.
 constexpr float LOG2E = 1.4426950408889634f;
+constexpr int LATENT_KC = 9, LATENT_VC = 16;
 
 template <int CT>   // tiles of 16 latent columns: rank <= 16 * CT
 __global__ __launch_bounds__(256) void latent_attention_bf16_kernel(
@@ -288,22 +289,44 @@ __global__ __launch_bounds__(256) void latent_attention_bf16_kernel(
   for (int c = 0; c < CT; ++c) acc[c] = floatx4{0.f, 0.f, 0.f, 0.f};
   const bf16x8 zero = {};
 
+  // the pages of a tile's keys are looked up a tile ahead: page_a / page_b of the keys whose kept rows this lane brings to the
+  // scores (key0 + col, key0 + 16 + col), page_v of the eight keys whose latent values it brings to the weighted sum
+  auto page_of = [&](int first_key, int last_key) -> int {
+    return last_key >= lo && first_key <= pos_last ? table[first_key / page_size] : -1;
+  };
+  int next_a = -1, next_b = -1, next_v = -1;
+  if (tile_begin < tile_end) {
+    next_a = page_of(tile_begin * 32 + col, tile_begin * 32 + col);
+    next_b = page_of(tile_begin * 32 + 16 + col, tile_begin * 32 + 16 + col);
+    next_v = page_of(tile_begin * 32 + 8 * g, tile_begin * 32 + 8 * g + 7);
+  }
+  constexpr int KC = LATENT_KC;      // products of 32 dims whose operands are asked for together: a wave waits for memory once a chunk
   for (int tile = tile_begin; tile < tile_end; ++tile) {
     const int key0 = tile * 32;
-    // scores: this lane brings the kept rows of keys key0 + col and key0 + 16 + col
     const int key_a = key0 + col, key_b = key_a + 16;
-    const int page_a = key_a >= lo && key_a <= pos_last ? table[key_a / page_size] : -1;
-    const int page_b = key_b >= lo && key_b <= pos_last ? table[key_b / page_size] : -1;
+    const int page_a = next_a, page_b = next_b, page_v = next_v;
+    if (tile + 1 < tile_end) {
+      next_a = page_of(key_a + 32, key_a + 32);
+      next_b = page_of(key_b + 32, key_b + 32);
+      next_v = page_of(key0 + 32 + 8 * g, key0 + 32 + 8 * g + 7);
+    }
     const bf16* row_a = pages + ((int64_t)(page_a < 0 ? 0 : page_a) * page_size + key_a % page_size) * width + g * 8;
     const bf16* row_b = pages + ((int64_t)(page_b < 0 ? 0 : page_b) * page_size + key_b % page_size) * width + g * 8;
     floatx4 s_a = {0.f, 0.f, 0.f, 0.f}, s_b = {0.f, 0.f, 0.f, 0.f};
-    for (int ks = 0; ks < width; ks += 32) {
-      const bool inside = ks + g * 8 < width;
-      const bf16x8 qf = inside && a_valid ? *(const bf16x8*)(q_row + ks) : zero;
-      const bf16x8 ka = inside && page_a >= 0 ? *(const bf16x8*)(row_a + ks) : zero;
-      const bf16x8 kb = inside && page_b >= 0 ? *(const bf16x8*)(row_b + ks) : zero;
-      s_a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf, ka, s_a, 0, 0, 0);
-      s_b = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf, kb, s_b, 0, 0, 0);
+    for (int ks = 0; ks < width; ks += 32 * KC) {
+      bf16x8 qf[KC], ka[KC], kb[KC];
+#pragma unroll
+      for (int u = 0; u < KC; ++u) {
+        const bool inside = ks + 32 * u + g * 8 < width;
+        qf[u] = inside && a_valid ? *(const bf16x8*)(q_row + ks + 32 * u) : zero;
+        ka[u] = inside && page_a >= 0 ? *(const bf16x8*)(row_a + ks + 32 * u) : zero;
+        kb[u] = inside && page_b >= 0 ? *(const bf16x8*)(row_b + ks + 32 * u) : zero;
+      }
+#pragma unroll
+      for (int u = 0; u < KC; ++u) {
+        s_a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[u], ka[u], s_a, 0, 0, 0);
+        s_b = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[u], kb[u], s_b, 0, 0, 0);
+      }
     }
     // the running softmax of the lane's four rows (a row's 32 scores lie in the 16 lanes that share g)
     float shrink[4];
@@ -338,17 +361,23 @@ __global__ __launch_bounds__(256) void latent_attention_bf16_kernel(
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     // the weighted sum: this lane brings, per tile of 16 columns, the latent values of column col at keys key0 + 8g .. + 7
     const int key_v = key0 + 8 * g;
-    const int page_v = key_v + 7 >= lo && key_v <= pos_last ? table[key_v / page_size] : -1;
     const bf16* column = value_pages + ((int64_t)(page_v < 0 ? 0 : page_v) * rank + col) * page_size + key_v % page_size;
     const bool rescale = shrink[0] != 1.f || shrink[1] != 1.f || shrink[2] != 1.f || shrink[3] != 1.f;
+    constexpr int VC = CT % LATENT_VC == 0 ? LATENT_VC : CT % 6 == 0 ? 6 : CT % 4 == 0 ? 4 : 2;      // column tiles whose values are asked for together
 #pragma unroll
-    for (int c = 0; c < CT; ++c) {
-      const bf16x8 vf = page_v >= 0 && 16 * c + col < rank ? *(const bf16x8*)(column + (int64_t)16 * c * page_size) : zero;
-      if (rescale) {
+    for (int c0 = 0; c0 < CT; c0 += VC) {
+      bf16x8 vf[VC];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[c][i] *= shrink[i];
+      for (int u = 0; u < VC; ++u)
+        vf[u] = page_v >= 0 && 16 * (c0 + u) + col < rank ? *(const bf16x8*)(column + (int64_t)16 * (c0 + u) * page_size) : zero;
+#pragma unroll
+      for (int u = 0; u < VC; ++u) {
+        if (rescale) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[c0 + u][i] *= shrink[i];
+        }
+        acc[c0 + u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf[u], acc[c0 + u], 0, 0, 0);
       }
-      acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf, acc[c], 0, 0, 0);
     }
   }
 

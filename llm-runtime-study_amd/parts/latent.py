@@ -29,7 +29,7 @@ import torch
 
 from ..kernels import ops
 from .attention import GQAAttention
-from .base import PagedKVNeed, Part, PartSpec, TensorSpec, create, register
+from .base import PagedKVNeed, Part, PartSpec, TensorSpec, create, length_class, register
 from .linear import linear, materialize, rows_of
 
 
@@ -149,6 +149,16 @@ class LatentAttention(Part):
         return linear(ctx, residual, heads_out.view(t, n * self.value_dim), self.w_o, accumulate=accumulate, then_norm=then_norm)
 
 
+    @staticmethod
+    def _splits_alone(workgroups: int, longest: int) -> int:
+        """Into how many workgroups the keys of a single token are divided: towards two workgroups a compute unit, at least
+        64 keys each (two tiles; a power of two that follows the length's class, so that eager steps and graph replays agree);
+        a workgroup walks its tiles one after the other, so a long context in few workgroups is a matter of latency."""
+        units = ops.compute_units()
+        if workgroups >= 2 * units:
+            return 1
+        return max(1, min(-(-2 * units // workgroups), length_class(longest) // 64, 64))
+
     def _attend_groups(self, ctx, latent, queries, gate, cache, group):
         """The matrix-core kernel: decode steps token by token, the single tokens at the head of a mixed step likewise, the
         rest by the step's query groups.  The keys of a group are divided between workgroups where the groups alone leave
@@ -163,10 +173,10 @@ class LatentAttention(Part):
             return (ctx.scratch(f"latent_{name}_o", (rows, n * splits * r), torch.float32), ctx.scratch(f"latent_{name}_ml", (rows, n * splits * 2), torch.float32))
 
         def alone(rows):
-            longest, bound = ctx.max_k if ctx.all_decode else ctx.max_k_bound, ctx.max_k_bound
+            longest = ctx.max_k if ctx.all_decode else ctx.max_k_bound
             if self.window is not None:
-                longest, bound = min(longest, self.window + 32), min(bound, self.window + 64)
-            splits = GQAAttention._decode_splits(rows * tiles, longest, bound, 1 << 20)
+                longest = min(longest, self.window + 32)
+            splits = self._splits_alone(rows * tiles, longest)
             part_o, part_ml = parts("single", rows, splits)
             ops.latent_attention_groups(latent[:rows], queries[:rows], cache.k_pages, cache.v_pages, group.block_table, ctx.token_slot, ctx.positions,
                                         None, None, 1, r, self.scale, sink=self.sink, gate=None if gate is None else gate[:rows], window=window,
