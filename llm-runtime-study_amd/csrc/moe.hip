@@ -237,7 +237,10 @@ __global__ __launch_bounds__(1024) void moe_route_align_kernel(const float* __re
   align_pairs(ids, tokens * top, experts, tile, sorted, capacity, place, tile_expert, max_tiles, shared);
 }
 
-enum { ACT_NONE = 0, ACT_RELU_SQUARED = 1 };
+// ACT_SILU_PAIRS: the matrix holds, for every feature j, a gate row 2j and an up row 2j + 1; the output has half as many columns,
+// out[:, j] = silu(gate_j) * up_j.  Every kernel below leaves a lane four neighbouring columns, so a lane holds whole pairs.
+enum { ACT_NONE = 0, ACT_RELU_SQUARED = 1, ACT_SILU_PAIRS = 2 };
+__device__ __forceinline__ float silu_times(float gate, float up) { return gate / (1.0f + expf(-gate)) * up; }
 
 // Any dtype, any shape: a 32 x 64 tile of outputs per workgroup of 256 threads, a thread 2 x 4 of them, each the
 // sum of its products in the order of k.
@@ -293,6 +296,10 @@ __global__ __launch_bounds__(256) void moe_experts_kernel(TO* __restrict__ out, 
       const int c = col0 + tx * 4 + jj;
       if (c >= n) continue;
       float v = acc[i][jj];
+      if (act == ACT_SILU_PAIRS) {
+        if (jj % 2 == 0) out[(int64_t)(row0 + m) * ldc + c / 2] = from_float<TO>(silu_times(v, acc[i][jj + 1]));
+        continue;
+      }
       if (act == ACT_RELU_SQUARED) v = v > 0.f ? v * v : 0.f;
       out[(int64_t)(row0 + m) * ldc + c] = from_float<TO>(v);
     }
@@ -377,6 +384,10 @@ __global__ __launch_bounds__(256) void moe_experts_bf16_kernel(TO* __restrict__ 
       for (int x = 0; x < 4; ++x) {
         if (c + x >= n) continue;
         float v = acc[i][jj][x];
+        if (act == ACT_SILU_PAIRS) {
+          if (x % 2 == 0) out[(int64_t)(row0 + m) * ldc + (c + x) / 2] = from_float<TO>(silu_times(v, acc[i][jj][x + 1]));
+          continue;
+        }
         if (act == ACT_RELU_SQUARED) v = v > 0.f ? v * v : 0.f;
         out[(int64_t)(row0 + m) * ldc + c + x] = from_float<TO>(v);
       }
@@ -464,6 +475,10 @@ __global__ __launch_bounds__(256) void moe_experts_bf16_wide_kernel(TO* __restri
       for (int x = 0; x < 4; ++x) {
         if (c + x >= n) continue;
         float v = acc[i][jj][x];
+        if (act == ACT_SILU_PAIRS) {
+          if (x % 2 == 0) out[(int64_t)(row0 + m) * ldc + (c + x) / 2] = from_float<TO>(silu_times(v, acc[i][jj][x + 1]));
+          continue;
+        }
         if (act == ACT_RELU_SQUARED) v = v > 0.f ? v * v : 0.f;
         out[(int64_t)(row0 + m) * ldc + c + x] = from_float<TO>(v);
       }
@@ -574,7 +589,11 @@ __global__ __launch_bounds__(256, 2) void moe_experts_bf16_fetch_kernel(TO* __re
 #pragma unroll
           for (int i = 0; i < 4; ++i) v[i] = v[i] > 0.f ? v[i] * v[i] : 0.f;
         }
-        if constexpr (sizeof(TO) == 2) *(bf16x4*)((bf16*)out + row_at + row0) = bf16x4{(bf16)v[0], (bf16)v[1], (bf16)v[2], (bf16)v[3]};
+        if (act == ACT_SILU_PAIRS) {
+          const float first = silu_times(v[0], v[1]), second = silu_times(v[2], v[3]);
+          if constexpr (sizeof(TO) == 2) *(bf16x2*)((bf16*)out + row_at + row0 / 2) = bf16x2{(bf16)first, (bf16)second};
+          else ((float*)out)[row_at + row0 / 2] = first, ((float*)out)[row_at + row0 / 2 + 1] = second;
+        } else if constexpr (sizeof(TO) == 2) *(bf16x4*)((bf16*)out + row_at + row0) = bf16x4{(bf16)v[0], (bf16)v[1], (bf16)v[2], (bf16)v[3]};
         else *(floatx4*)((float*)out + row_at + row0) = v;
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -582,10 +601,17 @@ __global__ __launch_bounds__(256, 2) void moe_experts_bf16_fetch_kernel(TO* __re
   }
 }
 
+// What becomes of a token's weighted sum y of its experts' rows:
+//   COMBINE_ADD        residual += y
+//   COMBINE_ADD_RMS    residual += w * y * rsqrt(mean(y^2) + eps)                       (a layer that normalises what a sublayer gives out)
+//   COMBINE_LAYERNORM  residual = w * (z - mean z) / sqrt(variance of z + eps), z = alpha * residual + y   (one that normalises the sum)
+enum { COMBINE_ADD = 0, COMBINE_ADD_RMS = 1, COMBINE_LAYERNORM = 2 };
+
 template <typename TW>
 __global__ __launch_bounds__(1024) void moe_combine_kernel(float* __restrict__ residual, const float* __restrict__ rows, int hidden,
                                                            const int* __restrict__ place, const float* __restrict__ weights, int top,
-                                                           const TW* __restrict__ norm_w, float eps, bf16* __restrict__ rounded) {
+                                                           const TW* __restrict__ norm_w, float eps, bf16* __restrict__ rounded, int kind,
+                                                           float alpha) {
   extern __shared__ float sum[];        // [hidden], 16 floats for the reduction, then the token's rows and weights [top] each
   float* share = sum + hidden + 16;
   int* where = (int*)(share + top);
@@ -595,21 +621,41 @@ __global__ __launch_bounds__(1024) void moe_combine_kernel(float* __restrict__ r
     where[c] = place[(int64_t)t * top + c];
   }
   __syncthreads();
+  float* out = residual + (int64_t)t * hidden;
   float ss = 0.f;
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
     float acc = 0.f;
     for (int c = 0; c < top; ++c) acc = fmaf(share[c], rows[(int64_t)where[c] * hidden + i], acc);
+    if (kind == COMBINE_LAYERNORM) {
+      acc = fmaf(alpha, out[i], acc);
+      ss += acc;                        // the sum of the row, for its mean
+    } else {
+      ss = fmaf(acc, acc, ss);
+    }
     sum[i] = acc;
-    ss = fmaf(acc, acc, ss);
   }
-  float* out = residual + (int64_t)t * hidden;
+  if (kind == COMBINE_LAYERNORM) {
+    const float mean = block_sum(ss, sum + hidden) / (float)hidden;
+    float sq = 0.f;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+      const float d = sum[i] - mean;    // written by this thread
+      sq = fmaf(d, d, sq);
+    }
+    const float inv = 1.0f / sqrtf(block_sum(sq, sum + hidden) / (float)hidden + eps);
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+      const float v = (sum[i] - mean) * inv * to_float(norm_w[i]);
+      out[i] = v;
+      if (rounded) rounded[(int64_t)t * hidden + i] = (bf16)v;
+    }
+    return;
+  }
   float inv = 1.f;
-  if (norm_w) {
+  if (kind == COMBINE_ADD_RMS) {
     ss = block_sum(ss, sum + hidden);
     inv = 1.0f / sqrtf(ss / (float)hidden + eps);
   }
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-    const float v = out[i] + (norm_w ? sum[i] * inv * to_float(norm_w[i]) : sum[i]);
+    const float v = out[i] + (kind == COMBINE_ADD_RMS ? sum[i] * inv * to_float(norm_w[i]) : sum[i]);
     out[i] = v;
     if (rounded) rounded[(int64_t)t * hidden + i] = (bf16)v;       // the stream as the next sublayer reads it
   }
@@ -684,13 +730,14 @@ LRS_API int lrs_moe_route_align(const float* logits, int ld, const float* bias, 
 }
 
 // out [max_tiles * tile, n] = rows of `a` (row pair / top of the sorted list if `gather`, else the sorted row
-// itself) times the tile's expert matrix w[expert] [n, k], transposed; act 1: the square of relu.
+// itself) times the tile's expert matrix w[expert] [n, k], transposed; act 1: the square of relu; act 2: see ACT_SILU_PAIRS (out has n / 2 columns).
 LRS_API int lrs_moe_experts(void* out, int out_dtype, int ldc, const void* a, const void* w, int dtype, int lda, int n, int k,
                             const int* sorted, const int* tile_expert, int max_tiles, int tile, int top, int gather, int act, void* stream) {
   LRS_REQUIRE(tile == GM || tile == WM, "moe_experts: tiles have %d or %d rows, got %d", GM, WM, tile);
   LRS_REQUIRE(max_tiles > 0 && n > 0 && k > 0 && top > 0, "moe_experts: bad sizes tiles=%d n=%d k=%d top=%d", max_tiles, n, k, top);
-  LRS_REQUIRE(lda >= k && ldc >= n, "moe_experts: strides lda=%d ldc=%d too small for k=%d n=%d", lda, ldc, k, n);
-  LRS_REQUIRE(act == ACT_NONE || act == ACT_RELU_SQUARED, "moe_experts: unknown activation %d", act);
+  LRS_REQUIRE(act == ACT_NONE || act == ACT_RELU_SQUARED || act == ACT_SILU_PAIRS, "moe_experts: unknown activation %d", act);
+  LRS_REQUIRE(lda >= k && ldc >= (act == ACT_SILU_PAIRS ? n / 2 : n), "moe_experts: strides lda=%d ldc=%d too small for k=%d n=%d", lda, ldc, k, n);
+  LRS_REQUIRE(act != ACT_SILU_PAIRS || n % 4 == 0, "moe_experts: pairs of gate and up rows come four rows at a time, got %d rows", n);
   hipStream_t s = (hipStream_t)stream;
   const bool cores = dtype == LRS_BF16 && k % GK == 0 && lda % 8 == 0 && ((uintptr_t)a % 16) == 0 && ((uintptr_t)w % 16) == 0;
   // large steps of shapes the fetching kernel takes: whole slices of 32 of K, rows of the output 16 bytes aligned, offsets
@@ -741,16 +788,19 @@ LRS_API int lrs_moe_experts(void* out, int out_dtype, int ldc, const void* a, co
 // residual [tokens, hidden] += (norm of) sum_c weights[t, c] * rows[place[t, c]]; norm_w null: the plain sum; rounded:
 // where the updated rows are left in bfloat16 as well, or null.
 LRS_API int lrs_moe_combine(float* residual, const float* rows, int tokens, int hidden, const int* place, const float* weights,
-                            int top, const void* norm_w, int norm_dtype, float eps, void* rounded, void* stream) {
+                            int top, const void* norm_w, int norm_dtype, float eps, void* rounded, int layer_norm, float alpha, void* stream) {
+  // layer_norm (with a norm weight): the stream becomes the layer norm of alpha * stream + sum, instead of taking the sum's RMS norm on top
   LRS_REQUIRE(tokens > 0 && hidden > 0 && top > 0, "moe_combine: bad sizes tokens=%d hidden=%d top=%d", tokens, hidden, top);
   LRS_REQUIRE(!norm_w || eps > 0.f, "moe_combine: eps must be positive");
+  LRS_REQUIRE(!layer_norm || norm_w, "moe_combine: a layer norm needs its weight");
+  const int kind = !norm_w ? COMBINE_ADD : layer_norm ? COMBINE_LAYERNORM : COMBINE_ADD_RMS;
   const size_t lds = (size_t)(hidden + 16 + 2 * top) * sizeof(float);
   LRS_REQUIRE(lds <= 64 * 1024, "moe_combine: a width of %d with %d choices is too much", hidden, top);
   hipStream_t s = (hipStream_t)stream;
   const int threads = hidden >= 2048 ? 1024 : 256;
   if (norm_w && norm_dtype == LRS_BF16)
-    moe_combine_kernel<bf16><<<tokens, threads, lds, s>>>(residual, rows, hidden, place, weights, top, (const bf16*)norm_w, eps, (bf16*)rounded);
+    moe_combine_kernel<bf16><<<tokens, threads, lds, s>>>(residual, rows, hidden, place, weights, top, (const bf16*)norm_w, eps, (bf16*)rounded, kind, alpha);
   else
-    moe_combine_kernel<float><<<tokens, threads, lds, s>>>(residual, rows, hidden, place, weights, top, (const float*)norm_w, eps, (bf16*)rounded);
+    moe_combine_kernel<float><<<tokens, threads, lds, s>>>(residual, rows, hidden, place, weights, top, (const float*)norm_w, eps, (bf16*)rounded, kind, alpha);
   return lrs_check_launch("moe_combine");
 }

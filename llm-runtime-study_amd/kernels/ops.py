@@ -169,7 +169,7 @@ _SIGNATURES = {
     "lrs_head_gemm": (c_int, [c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "lrs_latent_attention": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                      c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
-    "lrs_moe_combine": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p]),
+    "lrs_moe_combine": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_int, c_float, c_void_p]),
 }
 
 
@@ -1299,26 +1299,29 @@ def moe_route_align(logits: torch.Tensor, bias: torch.Tensor | None, ids: torch.
 
 
 def moe_experts(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, sorted_pairs: torch.Tensor, tile_expert: torch.Tensor, tile: int, top: int,
-                gather: bool, relu_squared: bool) -> None:
+                gather: bool, relu_squared: bool, silu_pairs: bool = False) -> None:
     """out [tiles * tile rows, N] = rows of `a` times w[expert of the tile] [N, K], transposed, for every tile in use.
     tile: rows of a tile, as moe_tile_rows() gave them for the step that was sorted.
-    gather: the row of a sorted pair is a[pair // top] (tokens); else `a` is in sorted order itself."""
+    gather: the row of a sorted pair is a[pair // top] (tokens); else `a` is in sorted order itself.
+    silu_pairs: w holds a gate row 2j and an up row 2j + 1 for every feature j, and out [*, N / 2] = silu(gate) * up."""
     experts, n, k = w.shape
     tiles = tile_expert.numel()
     _need(tile in (32, 128), "moe_experts: tiles have 32 or 128 rows")
     _need(w.is_contiguous() and a.dtype == w.dtype and a.shape[1] == k, "moe_experts: a [*, K] and w [E, N, K] must agree")
-    _need(out.shape == (tiles * tile, n) and out.dtype in (w.dtype, torch.float32), "moe_experts: out must be [tiles * tile rows, N]")
+    _need(not (relu_squared and silu_pairs) and (not silu_pairs or n % 4 == 0), "moe_experts: one activation, and pairs of rows four at a time")
+    _need(out.shape == (tiles * tile, n // 2 if silu_pairs else n) and out.dtype in (w.dtype, torch.float32), "moe_experts: out must be [tiles * tile rows, N] (N / 2 for pairs)")
     _need(gather or a.shape[0] >= tiles * tile, "moe_experts: sorted rows missing")
     _need(sorted_pairs.numel() >= tiles * tile, "moe_experts: sorted list too short")
     _launch("lrs_moe_experts", _dev(out, "out"), dtype_code(out.dtype), _rows(out, "out"), _dev(a, "a"), _dev(w, "w"), dtype_code(w.dtype),
             _rows(a, "a"), n, k, _dev(sorted_pairs, "sorted_pairs", torch.int32), _dev(tile_expert, "tile_expert", torch.int32), tiles, tile, top,
-            int(gather), int(relu_squared), _stream())
+            int(gather), 2 if silu_pairs else int(relu_squared), _stream())
 
 
 def moe_combine(residual: torch.Tensor, rows: torch.Tensor, place: torch.Tensor, weights: torch.Tensor, norm_weight: torch.Tensor | None,
-                eps: float = 0.0, rounded: torch.Tensor | None = None) -> None:
+                eps: float = 0.0, rounded: torch.Tensor | None = None, layer_norm_alpha: float | None = None) -> None:
     """residual [T, H] += sum over a token's choices of weights[t, c] * rows[place[t, c]]; with norm_weight: the RMS
-    norm (weight norm_weight, eps) of that sum instead of the sum itself.  rounded: bfloat16 [T, H] that receives the
+    norm (weight norm_weight, eps) of that sum instead of the sum itself; with layer_norm_alpha as well: residual becomes
+    the layer norm (norm_weight, eps) of layer_norm_alpha * residual + sum.  rounded: bfloat16 [T, H] that receives the
     updated rows as well."""
     tokens, top = weights.shape
     hidden = rows.shape[1]
@@ -1327,9 +1330,10 @@ def moe_combine(residual: torch.Tensor, rows: torch.Tensor, place: torch.Tensor,
     _need(place.dtype == torch.int32 and place.numel() >= tokens * top and place.is_contiguous() and weights.dtype == torch.float32
           and weights.is_contiguous(), "moe_combine: place must be int32 [T * top] and weights float32 [T, top]")
     _need(norm_weight is None or (norm_weight.numel() == hidden and norm_weight.is_contiguous()), "moe_combine: norm weight must hold H values")
+    _need(layer_norm_alpha is None or norm_weight is not None, "moe_combine: a layer norm needs its weight")
     _launch("lrs_moe_combine", _dev(residual, "residual"), _dev(rows, "rows"), tokens, hidden, _dev(place, "place"), _dev(weights, "weights"), top,
             None if norm_weight is None else _dev(norm_weight, "norm_weight"), 0 if norm_weight is None else dtype_code(norm_weight.dtype), eps,
-            _rounded(rounded, tokens, hidden, "moe_combine"), _stream())
+            _rounded(rounded, tokens, hidden, "moe_combine"), int(layer_norm_alpha is not None), 0.0 if layer_norm_alpha is None else layer_norm_alpha, _stream())
 
 
 # ------------------------------------------------------------------- latent attention

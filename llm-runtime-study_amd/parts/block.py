@@ -14,7 +14,8 @@ its output.
 PostNormBlock: the sublayers read the stream itself and each norm is applied to the sum, which replaces the stream:
     h = norm1(alpha * h + mixer(h));  h = norm2(alpha * h + feed_forward(h))      (the feed-forward may be absent)
 alpha is a constant of the model.  A sublayer writes into a float32 buffer of the step as for OutputNormBlock, and the norm's
-`scale_add_normed` does the rest in one kernel.
+`scale_add_normed` does the rest in one kernel; a feed-forward that says `applies_sum_norm` is given norm and alpha and does
+it in the kernel that sums its output up.
 """
 
 from __future__ import annotations
@@ -243,6 +244,11 @@ class PostNormBlock(OutputNormBlock):
         x = self._add_normed(ctx, self.mixer_norm, h, y, "stream_rounded_mid")
         if x is None:
             x = self._input(ctx, h)
+        if getattr(self.feed_forward, "applies_sum_norm", False) and getattr(self.ff_norm, "layer_parameters", None) is not None:
+            # the kernel that sums the feed-forward's output up takes the stream's share and the norm with it
+            rounded = ctx.scratch("stream_rounded_next", tuple(h.shape), torch.bfloat16) if ctx.dtype == torch.bfloat16 else None
+            self.feed_forward.forward(ctx, x, h, sum_norm=(self.ff_norm, self.alpha), rounded=rounded)
+            return rounded
         y = self._sublayer(ctx, self.feed_forward, x, h)
         return self._add_normed(ctx, self.ff_norm, h, y, "stream_rounded_next")
 

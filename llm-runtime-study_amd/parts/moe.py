@@ -11,7 +11,8 @@
 On the device: the router product, the choice per token, one sort of the step's (token, choice) pairs by expert
 into runs padded to whole row tiles, two grouped products over the sorted rows (the activation in the first one's
 epilogue), and one kernel that adds a token's rows up in the order of its choices, which can also apply the norm
-of a layer that normalises outputs and add the result into the stream (`applies_output_norm`).  Nothing is read
+of a layer that normalises outputs and add the result into the stream (`applies_output_norm`), or replace the stream by the
+layer norm of its sum with it (`applies_sum_norm`).  Nothing is read
 on the host: the launches are sized by the step's shape alone (at most pairs / tile + experts tiles).
 """
 
@@ -30,6 +31,7 @@ class RoutedExperts(Part):
     graph_safe = True
     plan_safe = True
     applies_output_norm = True    # forward(..., output_norm=norm): residual += norm(out) instead of residual += out
+    applies_sum_norm = True       # forward(..., sum_norm=(norm, alpha)): residual = norm(alpha * residual + out), for a layer norm
     rounds_stream = True          # forward(..., rounded=buffer): the updated stream is left there in bfloat16 as well
 
     def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int, top: int, router_bias: bool = False,
@@ -74,8 +76,10 @@ class RoutedExperts(Part):
             router = torch.cat((router, router.new_zeros(pad, self.hidden_size)), 0)
         self.router = router.contiguous()
         self.bias = weights[self.bias_name].float().contiguous() if self.router_bias else None
-        if self.gated:      # an expert's gate rows, then its up rows: one product makes both
-            self.up = torch.stack([torch.cat((weights[f"experts.{e}.gate.weight"], weights[f"experts.{e}.up.weight"]), 0).to(dtype)
+        if self.gated:      # a feature's gate row, then its up row: one product makes both, and its epilogue the gated activation
+            self.paired = self.intermediate_size % 2 == 0
+            join = (lambda g, u: torch.stack((g, u), 1).reshape(2 * self.intermediate_size, self.hidden_size)) if self.paired else (lambda g, u: torch.cat((g, u), 0))
+            self.up = torch.stack([join(weights[f"experts.{e}.gate.weight"], weights[f"experts.{e}.up.weight"]).to(dtype)
                                    for e in range(self.num_experts)]).contiguous()
         else:
             self.up = torch.stack([weights[f"experts.{e}.up.weight"].to(dtype) for e in range(self.num_experts)]).contiguous()
@@ -89,7 +93,7 @@ class RoutedExperts(Part):
     def flops(self, tokens, pairs):
         return 2.0 * tokens * (self.num_experts * self.hidden_size + (3 if self.gated else 2) * self.top * self.hidden_size * self.intermediate_size)
 
-    def forward(self, ctx, x, residual, then_norm=None, output_norm=None, rounded=None):
+    def forward(self, ctx, x, residual, then_norm=None, output_norm=None, rounded=None, sum_norm=None):
         t = rows_of(x)
         x = materialize(ctx, x)
         experts, top = self.num_experts, self.top
@@ -108,7 +112,9 @@ class RoutedExperts(Part):
             ops.moe_route(logits[:, :experts], self.bias, ids, weights, rule=self.rule)
             ops.moe_align(ids, experts, sorted_pairs, place, tile_expert)
         hidden = ctx.scratch("moe_hidden", (rows, self.intermediate_size), ctx.dtype)
-        if self.gated:
+        if self.gated and self.paired:
+            ops.moe_experts(hidden, x, self.up, sorted_pairs, tile_expert, tile, top, gather=True, relu_squared=False, silu_pairs=True)
+        elif self.gated:    # an odd size: gate rows then up rows, and the activation as a kernel of its own
             both = ctx.scratch("moe_gate_up", (rows, 2 * self.intermediate_size), ctx.dtype)
             ops.moe_experts(both, x, self.up, sorted_pairs, tile_expert, tile, top, gather=True, relu_squared=False)
             ops.silu_mul(hidden, both)
@@ -116,7 +122,10 @@ class RoutedExperts(Part):
             ops.moe_experts(hidden, x, self.up, sorted_pairs, tile_expert, tile, top, gather=True, relu_squared=True)
         outputs = ctx.scratch("moe_outputs", (rows, self.hidden_size), torch.float32)
         ops.moe_experts(outputs, hidden, self.down, sorted_pairs, tile_expert, tile, top, gather=False, relu_squared=False)
-        if output_norm is None:
+        if sum_norm is not None:
+            weight, eps = sum_norm[0].layer_parameters()
+            ops.moe_combine(residual[:t], outputs, place, weights, weight, eps, rounded=rounded, layer_norm_alpha=sum_norm[1])
+        elif output_norm is None:
             ops.moe_combine(residual[:t], outputs, place, weights, None, rounded=rounded)
         else:
             weight, eps = output_norm.rms_parameters()

@@ -89,6 +89,11 @@ class LayerNorm(Part):
     def bind(self, weights, dtype):
         self.weight = weights["weight"]
 
+    def layer_parameters(self):
+        """(weight, eps): says that this norm is w * (x - mean) / sqrt(variance + eps), so that the kernel that makes a
+        sublayer's output may apply it to the sum itself (a feed-forward that says `applies_sum_norm`)."""
+        return self.weight, self.eps
+
     def scale_add_normed(self, ctx, residual, y, alpha: float, rounded=None):
         ops.scale_add_layernorm(residual, y, alpha, self.weight, self.eps, rounded)
 
