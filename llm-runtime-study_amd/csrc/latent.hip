@@ -217,14 +217,20 @@ __global__ __launch_bounds__(256) void head_gemm_bf16_kernel(bf16* __restrict__ 
   const bf16* w_row = w + (int64_t)h * w_head + (int64_t)(n0 + col) * k + g * 8;
   floatx4 acc[4] = {};
   const bf16x8 zero = {};
-  for (int ks = 0; ks < k; ks += 32) {
-    const bool inside = ks + g * 8 < k;
-    const bf16x8 af = inside ? *(const bf16x8*)(a_row + ks) : zero;
+  constexpr int KC = 4;       // products of 32 inputs whose operands are asked for together
+  for (int ks = 0; ks < k; ks += 32 * KC) {
+    bf16x8 af[KC], wf[KC][4];
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const bf16x8 wf = inside && n0 + col + 16 * c < n ? *(const bf16x8*)(w_row + (int64_t)16 * c * k + ks) : zero;
-      acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, wf, acc[c], 0, 0, 0);
+    for (int u = 0; u < KC; ++u) {
+      const bool inside = ks + 32 * u + g * 8 < k;
+      af[u] = inside ? *(const bf16x8*)(a_row + ks + 32 * u) : zero;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) wf[u][c] = inside && n0 + col + 16 * c < n ? *(const bf16x8*)(w_row + (int64_t)16 * c * k + ks + 32 * u) : zero;
     }
+#pragma unroll
+    for (int u = 0; u < KC; ++u)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[u], wf[u][c], acc[c], 0, 0, 0);
   }
 #pragma unroll
   for (int c = 0; c < 4; ++c)
@@ -417,18 +423,33 @@ __global__ __launch_bounds__(256) void latent_attention_bf16_kernel(
 __global__ __launch_bounds__(256) void latent_merge_kernel(bf16* __restrict__ out, int out_stride, const float* __restrict__ part_o,
                                                            const float* __restrict__ part_ml, const float* __restrict__ sink,
                                                            const bf16* __restrict__ gate, int gate_stride, int heads, int rank, int splits) {
-  const int token = blockIdx.x, head = blockIdx.y;
+  __shared__ float weight[64];          // of each part: 2^(its maximum - the maximum of all), over the denominator, times the gate
+  const int token = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int64_t base = ((int64_t)token * heads + head) * splits;
-  float most = sink ? sink[head] * LOG2E : -INFINITY;
-  for (int s = 0; s < splits; ++s) most = fmaxf(most, part_ml[(base + s) * 2]);
-  float denominator = sink ? __builtin_amdgcn_exp2f(sink[head] * LOG2E - most) : 0.f;
-  for (int s = 0; s < splits; ++s) denominator += part_ml[(base + s) * 2 + 1] * __builtin_amdgcn_exp2f(part_ml[(base + s) * 2] - most);
-  float factor = 1.0f / denominator;
-  if (gate) factor *= 1.0f / (1.0f + expf(-(float)gate[(int64_t)token * gate_stride + head]));
-  for (int dim = threadIdx.x; dim < rank; dim += blockDim.x) {
+  if (lane < WAVE) {                    // the first wave: a part a lane (splits <= 64)
+    const float mine = lane < splits ? part_ml[(base + lane) * 2] : -INFINITY;
+    const float sum = lane < splits ? part_ml[(base + lane) * 2 + 1] : 0.f;
+    const float s2 = sink ? sink[head] * LOG2E : -INFINITY;
+    const float most = fmaxf(wave_max(mine), s2);
+    const float w = __builtin_amdgcn_exp2f(mine - most);
+    const float denominator = wave_sum(sum * w) + (sink ? __builtin_amdgcn_exp2f(s2 - most) : 0.f);
+    float factor = 1.0f / denominator;
+    if (gate) factor *= 1.0f / (1.0f + expf(-(float)gate[(int64_t)token * gate_stride + head]));
+    weight[lane] = w * factor;
+  }
+  __syncthreads();
+  constexpr int AT_ONCE = 8;            // parts whose sums are asked for together
+  for (int dim = lane; dim < rank; dim += blockDim.x) {
     float sum = 0.f;
-    for (int s = 0; s < splits; ++s) sum += part_o[(base + s) * rank + dim] * __builtin_amdgcn_exp2f(part_ml[(base + s) * 2] - most);
-    out[(int64_t)token * out_stride + (int64_t)head * rank + dim] = (bf16)(sum * factor);
+    for (int s0 = 0; s0 < splits; s0 += AT_ONCE) {
+      float o[AT_ONCE];
+#pragma unroll
+      for (int i = 0; i < AT_ONCE; ++i) o[i] = part_o[(base + (s0 + i < splits ? s0 + i : splits - 1)) * rank + dim];
+#pragma unroll
+      for (int i = 0; i < AT_ONCE; ++i)
+        if (s0 + i < splits) sum = fmaf(o[i], weight[s0 + i], sum);
+    }
+    out[(int64_t)token * out_stride + (int64_t)head * rank + dim] = (bf16)sum;
   }
 }
 
