@@ -42,9 +42,9 @@ def napizen_like(shape: dict, layers: int, experts: int = 32, top: int = 8, rank
     width, heads, dim = shape["hidden_size"], shape["num_attention_heads"], shape["head_dim"]
     ff = max(128, round(shape["intermediate_size"] / top / 128) * 128)
     mixer = {"heads": heads, "dim": dim, "rot_dim": rot, "vdim": dim, "kv_rank": rank, "scale": (dim + rot) ** -0.5,
-             "rot": {"base": 1000000.0, "dims": rot, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+             "rot": {"base": 500000.0, "dims": rot, "scaling": {"factor": 8.0, "original": 8192, "fast": 24.0, "slow": 2.0}}}
     dense = {"kind": "dense", "ff": shape["intermediate_size"]}
     routed = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top, "scale": 2.5, "groups": {"count": 8, "keep": 4}}}
     return {"architecture": "Napizen", "vocab": shape["vocab_size"], "width": width, "norm": {"eps": 1e-6}, "postln_alpha": 2.0,
-            "embedding": {"scale": 1.0}, "logit_softcap": 30.0,
+            "embedding": {"scale": 1.0}, "logit_softcap": 50.0,
             "layers": [{"type": "latent_attention", "mixer": mixer, "mlp": routed if index % 2 else dense} for index in range(layers)]}

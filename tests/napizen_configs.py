@@ -37,7 +37,7 @@ def model(vocab, width, eps, alpha, layers, embedding=1.0, cap=None):
 MIXED = model(211, 64, 1e-5, 1.7, [
     latent(3, 16, 8, 24, 40, 0.2, 10000.0, (8.0, 64, 16.0, 2.0), dense(96)),
     latent(2, 24, 4, 8, 20, 0.31, 500.0, None, experts(32, 6, 2, 1.5, (2, 1))),
-    latent(4, 8, 12, 16, 32, 0.25, 1e6, (4.0, 256, 32.0, 1.0), None),
+    latent(4, 8, 12, 16, 32, 0.25, 2e5, (5.0, 256, 20.0, 1.0), None),
     latent(3, 16, 8, 24, 40, 0.2, 10000.0, (8.0, 64, 16.0, 2.0), experts(24, 9, 3, 2.5, (3, 2))),
 ], embedding=6.0, cap=9.0)
 # values that coincide or are 1: one head, groups of one expert, every group kept, one choice, alpha 1, no cap, a rotated part
@@ -50,12 +50,12 @@ PLAIN = model(157, 48, 3e-6, 1.0, [
 ])
 # sizes the matrix-core kernels take: rows of 128 and 160 kept values, heads of 64 and 128, eight and sixteen heads
 CORES = model(300, 128, 1e-6, 2.0, [
-    latent(8, 64, 32, 64, 96, 0.1, 1e6, (4.0, 128, 32.0, 1.0), dense(256)),
-    latent(16, 32, 16, 32, 64, 0.14, 1e4, None, experts(64, 8, 2, 2.0, (4, 3))),
+    latent(8, 64, 32, 64, 96, 0.1, 3e5, (6.0, 128, 24.0, 1.5), dense(256)),
+    latent(16, 32, 16, 32, 64, 0.14, 1e4, None, experts(64, 8, 3, 1.5, (4, 2))),
     latent(4, 128, 32, 128, 128, 0.08, 1e5, (16.0, 64, 8.0, 2.0), experts(128, 4, 4, 1.0)),
 ], embedding=11.0, cap=25.0)
 # wide enough that prompts go through the products for many rows
 WIDE = model(1000, 512, 1e-6, 3.0, [
-    latent(8, 64, 32, 64, 128, 0.1, 1e6, (4.0, 512, 32.0, 1.0), experts(256, 8, 2, 2.0, (4, 2))),
+    latent(8, 64, 32, 64, 128, 0.1, 5e5, (3.0, 512, 28.0, 1.0), experts(256, 8, 2, 1.25, (4, 2))),
     latent(8, 64, 64, 128, 192, 0.09, 1e4, None, dense(1024)),
-], embedding=22.0, cap=30.0)
+], embedding=22.0, cap=28.0)

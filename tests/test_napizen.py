@@ -87,8 +87,8 @@ def test_configurations_that_cannot_run_are_refused(broken, message):
         config_from_dict(raw)
 
 
-@pytest.mark.parametrize("dims,base,scaling", [(8, 10000.0, (8.0, 64, 16.0, 2.0)), (12, 1e6, (4.0, 256, 32.0, 1.0)), (64, 1e4, (40.0, 4096, 32.0, 1.0)),
-                                               (16, 1e6, (4.0, 2048, 32.0, 1.0)), (2, 30.0, (3.0, 10, 2.0, 1.0)), (32, 500.0, None)])
+@pytest.mark.parametrize("dims,base,scaling", [(8, 10000.0, (8.0, 64, 16.0, 2.0)), (12, 2e5, (5.0, 256, 20.0, 1.0)), (64, 1e4, (40.0, 4096, 32.0, 1.0)),
+                                               (16, 2e5, (6.0, 1024, 24.0, 2.0)), (2, 30.0, (3.0, 10, 2.0, 1.0)), (32, 500.0, None)])
 def test_stretched_frequencies(dims, base, scaling):
     """The position part's frequencies and magnitude against the plain implementation's; where the blend begins and ends."""
     from llm_runtime_study_amd.parts import PartSpec, create
