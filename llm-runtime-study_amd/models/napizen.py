@@ -54,6 +54,8 @@ def build_spec(config: NapizenConfig) -> ModelSpec:
         if layer.mlp is not None:
             params["feed_forward"] = _feed_forward(config, layer)
             params["ff_norm"] = norm
+        else:
+            params["norm_without_ff"] = norm      # asked for as optional: see PostNormBlock
         layers.append(PartSpec("postnorm", params))
     return ModelSpec(
         architecture=NapizenConfig.ARCHITECTURE, vocab_size=config.vocab_size, hidden_size=config.width, layers=tuple(layers),

@@ -213,9 +213,16 @@ class PostNormBlock(OutputNormBlock):
     buffer a sublayer writes, what is handed to the next block) is OutputNormBlock's."""
 
     def __init__(self, mixer: PartSpec, mixer_norm: PartSpec, feed_forward: PartSpec | None = None, ff_norm: PartSpec | None = None,
-                 alpha: float = 1.0, names: dict | None = None):
+                 alpha: float = 1.0, names: dict | None = None, norm_without_ff: PartSpec | None = None):
         if (feed_forward is None) != (ff_norm is None):
             raise ValueError("a feed-forward and its norm come together")
+        if norm_without_ff is not None and feed_forward is not None:
+            raise ValueError("norm_without_ff is for a layer that has no feed-forward")
+        # A layer without feed-forward has no second update.  Checkpoints that carry the second norm's weight for such a
+        # layer all the same mean h = norm2(alpha * h) by it: the tensor is asked for as optional, and the update is made
+        # exactly when it was there.
+        self.norm_without_ff = None if norm_without_ff is None else create("norm", norm_without_ff)
+        self.norm_without_ff_bound = False
         self.alpha = float(alpha)
         self.mixer = create("mixer", mixer)
         self.mixer_norm = create("norm", mixer_norm)
@@ -226,6 +233,23 @@ class PostNormBlock(OutputNormBlock):
                 raise ValueError("a norm of the sum of stream and sublayer must offer scale_add_normed(ctx, residual, y, alpha)")
         self.names = {"mixer": "mixer", "feed_forward": "feed_forward", "mixer_norm": "mixer_norm", "ff_norm": "ff_norm"}
         self.names.update(names or {})
+
+    def tensors(self):
+        out = super().tensors()
+        if self.norm_without_ff is not None:
+            from dataclasses import replace
+
+            out.update({f"{self.names['ff_norm']}.{name}": replace(spec, optional=True) for name, spec in self.norm_without_ff.tensors().items()})
+        return out
+
+    def bind(self, weights, dtype):
+        super().bind(weights, dtype)
+        if self.norm_without_ff is not None:
+            prefix = self.names["ff_norm"] + "."
+            wanted = list(self.norm_without_ff.tensors())
+            self.norm_without_ff_bound = bool(wanted) and all(prefix + name in weights for name in wanted)
+            if self.norm_without_ff_bound:
+                self.norm_without_ff.bind(under(weights, prefix), dtype)
 
     def _add_normed(self, ctx, norm, h, y, name):
         """h = norm(alpha * h + y); returns the new stream as the next reader's activation if the norm's kernel left it."""
@@ -239,9 +263,11 @@ class PostNormBlock(OutputNormBlock):
     def forward(self, ctx, h, cache, given=None):
         x = given if given is not None else self._input(ctx, h)
         y = self._sublayer(ctx, self.mixer, x, h, cache)
-        if self.feed_forward is None:
+        if self.feed_forward is None and not self.norm_without_ff_bound:
             return self._add_normed(ctx, self.mixer_norm, h, y, "stream_rounded_next")
         x = self._add_normed(ctx, self.mixer_norm, h, y, "stream_rounded_mid")
+        if self.feed_forward is None:       # the second norm's weight was there: h = norm2(alpha * h + 0)
+            return self._add_normed(ctx, self.norm_without_ff, h, self._cleared(ctx, h), "stream_rounded_next")
         if x is None:
             x = self._input(ctx, h)
         if getattr(self.feed_forward, "applies_sum_norm", False) and getattr(self.ff_norm, "layer_parameters", None) is not None:

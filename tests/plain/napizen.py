@@ -155,6 +155,8 @@ def forward(weights: dict, raw: dict, ids, streams: list | None = None) -> torch
             f = under(w, "mlp.")
             y = gated_ff(x, f["gate"], f["up"], f["down"]) if mlp["kind"] == "dense" else routed_ff(x, f, mlp)
             x = centred_norm(alpha * x + y, w["norm2"], eps)
+        elif "norm2" in w:          # a layer without feed-forward whose second norm is stored all the same: nothing is added
+            x = centred_norm(alpha * x, w["norm2"], eps)
         if streams is not None:
             streams.append(x.clone())
     logits = centred_norm(x, weights["final.norm"], eps) @ weights["head"].T

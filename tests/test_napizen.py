@@ -31,8 +31,8 @@ def test_configuration_reads_back_and_names_its_tensors(tmp_path):
             assert names[p + "mix.sink"].shape == (m["heads"],) and names[p + "mix.g"].shape == (m["heads"], raw["width"])
             assert names[p + "mix.o"].shape == (raw["width"], m["heads"] * m["vdim"])
             mlp = layer["mlp"]
-            if mlp is None:
-                assert p + "norm2" not in names and not any(name.startswith(p + "mlp.") for name in names)
+            if mlp is None:      # no second update; the second norm's weight is taken if a checkpoint has it all the same
+                assert names[p + "norm2"].optional and not any(name.startswith(p + "mlp.") for name in names)
             elif mlp["kind"] == "dense":
                 assert names[p + "mlp.gate"].shape == names[p + "mlp.up"].shape == (mlp["ff"], raw["width"]) and names[p + "mlp.down"].shape == (raw["width"], mlp["ff"])
             else:
@@ -45,6 +45,10 @@ def test_configuration_reads_back_and_names_its_tensors(tmp_path):
         assert model.graph_safe() and model.plan_safe()
     folder = configs.write_folder(configs.MIXED, 3, tmp_path / "m")
     assert load_config(folder).to_json_dict() == configs.MIXED
+    from tests.plain import napizen as plain_model
+
+    stored = plain_model.load_model_dir(folder)[1]
+    assert "l2.norm1" in stored and "l2.norm2" not in stored and "l1.norm2" in stored       # folders of random weights leave it out
 
 
 def test_what_the_file_leaves_out_does_not_exist():

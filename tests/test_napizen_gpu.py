@@ -437,6 +437,30 @@ def test_a_wider_model_through_the_products_for_many_rows(tmp_path, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_layer_without_feed_forward_whose_second_norm_is_stored(tmp_path, dtype):
+    """Such a layer has no second update, and folders of random weights hold no second norm for it.  A checkpoint that holds
+    one all the same is taken to mean h = norm2(alpha * h): both kinds of folder against the plain implementation."""
+    raw = configs.MIXED
+
+    def edit(tensors):
+        tensors["l2.norm2"] = (tensors["l2.norm1"].float() * 0.7 + 0.4).to(torch.bfloat16)
+
+    rng = np.random.default_rng(13)
+    requests = {"p": rng.integers(0, raw["vocab"], 70).tolist(), "q": rng.integers(0, raw["vocab"], 33).tolist()}
+    rows = {}
+    for name, change in (("without", None), ("with", edit)):
+        folder = configs.write_folder(raw, 71, tmp_path / name, change)
+        _, weights = plain.load_model_dir(folder)
+        assert ("l2.norm2" in weights) == (change is not None)
+        want = {key: plain.forward(weights, raw, tokens) for key, tokens in requests.items()}
+        steps = traces.portions(requests, sizes=(9, 2, 30, 1, 1))
+        got = traces.collect(steps, run_replay(folder, dtype, steps, 128, tmp_path / f"o_{name}"), raw["vocab"])
+        check(got, want, dtype)
+        rows[name] = want["p"][-1]
+    assert (rows["with"] - rows["without"]).norm() > 0.05 * rows["without"].norm()      # the stored norm matters
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding(models, dtype, tmp_path):
     """A prompt of 20 tokens and 300 more one by one, beside a second request that starts later."""
     folder, raw, _, _ = models["mixed"]
